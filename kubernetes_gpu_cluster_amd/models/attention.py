@@ -190,3 +190,55 @@ class LatentAttention(nn.Module):
                                  w.size if w else 0, 0, None)                  # [T, H * rank]
         o = torch.bmm(o.view(T, H, rank).transpose(0, 1), self.w_uv)           # [H, T, dv]
         return self.o_proj(ops.gate_mul(o.transpose(0, 1), proj[:, self.n_q + self.n_kv:]))
+
+
+class AttentionCore(nn.Module):
+    """The part of a softmax attention mixer between its projections, for mixers whose
+    projections are merged with a neighbour's (a parallel mixer): reads q | k | v (| the
+    gate pre-activation) from columns ``col0 ..`` of a wider projection, rotates q and k
+    (pairs (i, i + dims/2), or (2i, 2i + 1) when ``spec.rotary.interleaved``), stores k and
+    v in the paged cache chosen at call time, attends causally (``spec.window`` when set)
+    with scores q.k * scale that pass cap * tanh(. / cap) when ``spec.softcap`` > 0,
+    multiplies the concatenated heads by sigmoid of the gate columns (``spec.elem_gate``)
+    and by ``out_scale``, and writes them into a column slice of the output projection's
+    input.  Softmax, scores and rotation are fp32."""
+
+    def __init__(self, spec, out_scale: float = 1.0):
+        super().__init__()
+        self.spec, self.out_scale = spec, float(out_scale)
+        H, G, dk, dv = spec.heads, spec.kv_heads, spec.dim, spec.vdim
+        assert H % G == 0, "query heads must be a multiple of key/value heads"
+        assert spec.rot_dims % 2 == 0 and spec.rot_dims <= dk
+        self.n_qkv = H * dk + G * dk + G * dv
+        self.n_in = self.n_qkv + (H * dv if spec.elem_gate else 0)
+        self.n_out = H * dv
+        self.scale = spec.dim ** -0.5 if spec.scale is None else spec.scale
+        self.rope = None            # [max_pos, rot_dims] fp32, set by prepare()
+
+    def prepare(self, tables: dict, max_pos: int, device) -> None:
+        sp = self.spec
+        if not sp.rot_dims:
+            return
+        key = (sp.rot_dims, sp.rot_base)
+        if key not in tables:
+            tables[key] = ops.ref.rope_table(sp.rot_dims, max_pos, sp.rot_base).to(device)
+        self.rope = tables[key]
+
+    def forward(self, proj: torch.Tensor, col0: int, positions: torch.Tensor,
+                ctx: ForwardContext, cache_idx: int, out: torch.Tensor) -> None:
+        sp = self.spec
+        kc, vc = ctx.kv_caches[cache_idx]
+        qkv = proj[:, col0: col0 + self.n_qkv]
+        q = ops.rope_kv_store(qkv, positions, self.rope, kc, vc, ctx.attn.slot_mapping,
+                              sp.heads, sp.kv_heads, sp.dim, sp.vdim,
+                              bool(sp.rotary and sp.rotary.interleaved))
+        w = sp.window
+        if not sp.elem_gate:
+            ops.window_attention(q, kc, vc, positions, ctx.attn, self.scale,
+                                 w.size if w else 0, w.keep_first if w else 0, None,
+                                 sp.softcap, self.out_scale, out=out)
+            return
+        o = ops.window_attention(q, kc, vc, positions, ctx.attn, self.scale,
+                                 w.size if w else 0, w.keep_first if w else 0, None, sp.softcap)
+        g = proj[:, col0 + self.n_qkv: col0 + self.n_in]
+        ops.gate_mul(o.view(o.shape[0], sp.heads, sp.vdim), g, self.out_scale, out=out)

@@ -54,6 +54,12 @@ class FeedForwardSpec:
     top: int = 0
     route_scale: float = 1.0
     shared_ff: int = 0
+    # gated: down(act(gate h) * up h); not gated: down(act(up h)).  None: the kind's usual
+    # form (dense: gated, moe: ungated)
+    gated: Optional[bool] = None
+    # "sigmoid": the routing described above; "softmax": logits W_r h + b_r, the ``top``
+    # largest chosen, their weights the softmax over the chosen logits only
+    router: str = "sigmoid"
 
 
 @dataclasses.dataclass(frozen=True)
@@ -70,7 +76,17 @@ class MixerSpec:
     unrotated dimensions plus ``rot_dims`` rotated ones, the rotated key part shared by
     all heads.  The paged cache holds the latent and the rotated key part only.
     kind "mingru": an element-wise gated recurrence of ``width`` channels (one fp32 state
-    vector per sequence) with a SiLU output gate."""
+    vector per sequence) with a SiLU output gate.
+    kind "parallel": two mixers side by side on the same input, ``left`` (an "attention"
+    spec) and ``right`` (a "mamba2" or "gated_delta" spec); the result is
+    left_scale * left + right_scale * right.
+    kind "mamba2": the state-space-duality recurrence, ``heads`` heads of ``vdim`` channels
+    with a [dim, vdim] fp32 state each (dim: the state size N), B / C shared by the heads
+    of one of ``kv_heads`` groups, a causal convolution of ``conv`` taps with bias on
+    x | B | C, a SiLU gate before an RMS norm in ``inner_norm_groups`` parts.
+    kind "gated_delta": the gated delta rule, ``heads`` value heads over ``kv_heads``
+    query / key heads, a [dim, vdim] fp32 state per head, convolutions of ``conv`` taps
+    without bias on q, k and v, a per-head RMS norm and a SiLU gate after it."""
     kind: str
     heads: int
     dim: int
@@ -88,6 +104,18 @@ class MixerSpec:
     width: int = 0               # mingru: recurrent channels
     rotary: Optional[RotarySpec] = None     # latent_attention (rot_dims = rotary.dims)
     mlp: Optional[FeedForwardSpec] = None   # feed-forwards other than the plain dense one
+    # attention inside a parallel mixer: biases on q, k, v and the output projection, a
+    # tanh cap on the scaled scores (0: none), an element-wise sigmoid gate sigmoid(W_g h)
+    # on the concatenated heads; ``rotary.interleaved`` chooses the pair layout
+    bias: bool = False
+    softcap: float = 0.0
+    elem_gate: bool = False
+    conv: int = 0                # mamba2 / gated_delta: taps of the causal convolution
+    inner_norm_groups: int = 1   # mamba2: parts of the gated RMS norm
+    left: Optional["MixerSpec"] = None      # parallel
+    right: Optional["MixerSpec"] = None
+    left_scale: float = 1.0
+    right_scale: float = 1.0
 
     @property
     def is_attention(self) -> bool:
@@ -138,6 +166,10 @@ class ModelConfig:
     layer_loop: Optional[tuple] = None
     side_dim: int = 0
     token_shift: bool = False
+    # arch "nolesun": every sublayer's result is RMS-normed and scaled per channel before
+    # it joins the stream (norm weights stored around zero); before each pass of the loop
+    # x <- W_in [x; embedding output] + step[pass]
+    loop_mix: bool = False
 
     @property
     def q_size(self) -> int:
@@ -178,6 +210,14 @@ class ModelConfig:
                     n += sp.kv_rank * sp.heads * (sp.dim + sp.vdim) + 2 * h * sp.heads * sp.vdim
                 elif sp.kind == "mingru":
                     n += 4 * h * sp.width
+                elif sp.kind == "parallel":
+                    l, r = sp.left, sp.right
+                    n += h * (l.heads * l.dim + l.kv_heads * (l.dim + l.vdim))
+                    n += l.heads * l.vdim * h * (2 if l.elem_gate else 1)
+                    if r.kind == "mamba2":
+                        n += h * (3 * r.heads * r.vdim + 2 * r.kv_heads * r.dim + r.heads)
+                    else:
+                        n += h * (2 * r.kv_heads * r.dim + 3 * r.heads * r.vdim + 2 * r.heads)
                 elif sp.kind == "attention":
                     n += h * (sp.heads * sp.dim + sp.kv_heads * (sp.dim + sp.vdim) + sp.heads)
                 else:
@@ -188,9 +228,10 @@ class ModelConfig:
                 if f is None:
                     n += 2 * h * sp.ff
                 elif f.kind == "dense":
-                    n += 3 * h * f.ff
+                    n += (2 if f.gated is False else 3) * h * f.ff
                 else:
-                    n += 2 * h * (f.experts * f.ff + f.shared_ff) + h * (f.experts + 1)
+                    n += ((3 if f.gated else 2) * h * f.experts * f.ff + 2 * h * f.shared_ff
+                          + h * (f.experts + 1))
                 n += 2 * h * self.side_dim
             return n + self.vocab_size * self.side_dim * len(self.layer_specs)
         attn = h * (self.q_size + 2 * self.kv_size) + self.q_size * h
@@ -208,9 +249,11 @@ class ModelConfig:
             n = {i: 0 for i in range(len(self.layer_specs))}
             for i, _ in self.layer_runs():
                 n[i] += 1
+            att = [(i, sp.left if sp.kind == "parallel" else sp)
+                   for i, sp in enumerate(self.layer_specs) if sp.is_attention or sp.kind == "parallel"]
             return sum(n[i] * dtype_bytes * (sp.kv_rank + sp.rot_dims if sp.kind == "latent_attention"
                                              else sp.kv_heads * (sp.dim + sp.vdim))
-                       for i, sp in enumerate(self.layer_specs) if sp.is_attention)
+                       for i, sp in att)
         return 2 * self.num_layers * self.num_kv_heads * self.head_dim * dtype_bytes
 
     def shrink(self, **kw) -> "ModelConfig":
@@ -467,8 +510,77 @@ def konovik_config(d: dict, name: str) -> ModelConfig:
         bos_token_id=int(d.get("bos_token_id", 0)), eos_token_id=int(d.get("eos_token_id", -1)))
 
 
+def _nolesun_ff(mlp: Optional[dict]) -> Optional[FeedForwardSpec]:
+    if not mlp:
+        return None
+    kind = mlp.get("kind", "dense")
+    if kind == "dense":
+        return FeedForwardSpec("dense", int(mlp["ff"]), act="relu2", gated=False)
+    if kind == "moe":
+        rt = mlp["router"]
+        return FeedForwardSpec("moe", int(mlp["expert"]["ff"]), act="silu", gated=True,
+                               experts=int(rt["experts"]), top=int(rt["top"]), router="softmax")
+    raise ValueError(f"unsupported feed-forward kind {kind!r}")
+
+
+def _nolesun_spec(entry: dict) -> MixerSpec:
+    """One entry of a Nolesun ``layers`` list.  Type "parallel": attention (pairs
+    (i, i + dims/2)) beside Mamba-2; type "parallel_2": attention with biases, pairs
+    (2i, 2i + 1), a score cap and an element-wise output gate beside the gated delta rule."""
+    kind, m = entry["type"], entry["mixer"]
+    if kind not in ("parallel", "parallel_2"):
+        raise ValueError(f"unknown mixer type {kind!r}")
+    two = kind == "parallel_2"
+    mlp = _nolesun_ff(entry.get("mlp"))
+    l, r = m["left"], m["right"]
+    rot = l.get("rot")
+    rs = (RotarySpec(int(rot["dims"]), float(rot["base"]), interleaved=two)
+          if rot and int(rot["dims"]) else None)
+    H = int(l["heads"])
+    left = MixerSpec("attention", H, int(l["dim"]), int(l["vdim"]),
+                     kv_heads=int(l.get("kv_heads", H)), scale=float(l["scale"]),
+                     rot_dims=rs.dims if rs else 0, rot_base=rs.base if rs else 10000.0,
+                     rotary=rs, bias=two, softcap=float(l.get("softcap", 0.0)) if two else 0.0,
+                     elem_gate=two)
+    Hr = int(r["heads"])
+    if two:
+        right = MixerSpec("gated_delta", Hr, int(r["dim"]), int(r["vdim"]),
+                          kv_heads=int(r.get("kv_heads", Hr)), conv=int(r["conv"]))
+    else:
+        right = MixerSpec("mamba2", Hr, int(r["state"]), int(r["vdim"]),
+                          kv_heads=int(r.get("groups", 1)), conv=int(r["conv"]),
+                          inner_norm_groups=int(r.get("norm_groups", 1)))
+    if left.heads % left.kv_heads or right.heads % right.kv_heads:
+        raise ValueError("heads must be a multiple of the key/value heads (groups)")
+    return MixerSpec("parallel", H, left.dim, left.vdim, kv_heads=left.kv_heads,
+                     ff=mlp.ff if mlp else 0, mlp=mlp, left=left, right=right,
+                     left_scale=float(m.get("left_scale", 1.0)),
+                     right_scale=float(m.get("right_scale", 1.0)))
+
+
+def nolesun_config(d: dict, name: str) -> ModelConfig:
+    """A Nolesun config.json (``architecture``, ``width``, ``vocab``, ``layers``, ``loop``,
+    ``norm``, ``embedding``) -> ModelConfig."""
+    specs = tuple(_nolesun_spec(e) for e in d["layers"])
+    lp = d.get("loop")
+    loop = (int(lp["start"]), int(lp["stop"]), int(lp["times"])) if lp else None
+    if loop and not (0 <= loop[0] < loop[1] <= len(specs) and loop[2] >= 1):
+        raise ValueError(f"bad layer loop {loop}")
+    a = specs[0].left
+    return ModelConfig(
+        name, "nolesun", len(specs), int(d["width"]), a.heads, a.kv_heads, a.dim,
+        max((sp.ff for sp in specs), default=0), int(d["vocab"]),
+        max_position=int(d.get("max_position", 8192)), rope_theta=a.rot_base,
+        rms_eps=float(d["norm"]["eps"]), layer_specs=specs,
+        embed_scale=float(d.get("embedding", {}).get("scale", 1.0)), layer_loop=loop,
+        loop_mix=loop is not None,
+        bos_token_id=int(d.get("bos_token_id", 0)), eos_token_id=int(d.get("eos_token_id", -1)))
+
+
 def _from_hf_config(d: dict, name: str) -> ModelConfig:
     """Map an HF config.json dict onto ModelConfig."""
+    if d.get("architecture") == "Nolesun":
+        return nolesun_config(d, name)
     if d.get("architecture") == "Dilavik":
         return dilavik_config(d, name)
     if d.get("architecture") == "Konovik":

@@ -319,3 +319,43 @@ class SigmoidRoutedExperts(nn.Module):
         if routed is not None and shared is None:
             return routed
         return ops.moe_finish(routed, dense, topk_w, topk_ids, shared, gate)
+
+
+class SoftmaxRoutedExperts(nn.Module):
+    """Mixture of gated experts down(silu(gate h) * up h) with softmax routing: logits
+    W_r h + b_r in fp32; the ``top`` largest are chosen and weighted by the softmax over the
+    chosen logits only.  Expert weights are kept as w13 [E, 2 ff, hidden] (gate rows, then
+    up rows) and w2 [E, hidden, ff].
+
+    Expert GEMMs: the grouped MFMA GEMM over expert-sorted rows (``ops.fused_moe``) where
+    its tiles cover the shapes (16-bit activations, 2 ff % 128 == 0, hidden % 128 == 0,
+    ff % 64 == 0); otherwise every expert runs on every token as one batched GEMM pair and
+    the chosen outputs are gathered -- no host synchronisation either way, so decode graphs
+    capture the block.  One GPU per replica."""
+
+    def __init__(self, hidden: int, spec, dtype, device):
+        super().__init__()
+        assert spec.act == "silu" and spec.gated and spec.router == "softmax"
+        self.spec = spec
+        E, I = spec.experts, spec.ff
+        z = lambda *s: nn.Parameter(torch.zeros(*s, dtype=dtype, device=device),   # noqa: E731
+                                    requires_grad=False)
+        self.w13 = z(E, 2 * I, hidden)
+        self.w2 = z(E, hidden, I)
+        self.router = z(E, hidden)
+        self.router_bias = nn.Parameter(torch.zeros(E, dtype=torch.float32, device=device),
+                                        requires_grad=False)
+        self.native = (torch.device(device).type == "cuda" and dtype != torch.float32 and
+                       ops.moe_supported(2 * I, hidden) and ops.moe_supported(hidden, I))
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        sp = self.spec
+        logits = ops.gate_proj(x, self.router, self.router_bias, ops.GATE_NONE)    # fp32 [T, E]
+        topk_w, topk_ids = ops.moe_topk_softmax(logits, sp.top)
+        if self.native and x.is_cuda:
+            return ops.fused_moe(x, self.w13, self.w2, topk_w, topk_ids)
+        T = x.shape[0]
+        xe = x.unsqueeze(0).expand(sp.experts, T, x.shape[1])
+        a = ops.silu_mul(torch.bmm(xe, self.w13.transpose(1, 2)))
+        dense = torch.bmm(a, self.w2.transpose(1, 2))
+        return ops.moe_finish(None, dense, topk_w, topk_ids, None, None)

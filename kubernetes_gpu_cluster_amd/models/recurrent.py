@@ -84,3 +84,85 @@ class MinGRUMixer(nn.Module):
         y = ops.mingru_scan(self.zxg_proj(h), self.zx_bias, state, ctx.attn, self.spec.width,
                             h.dtype)
         return self.o_proj(y)
+
+
+class Mamba2Core(nn.Module):
+    """The Mamba-2 (state-space duality) mixer between its projections.  Its projection
+    columns are z | x | B | C | dt (inner = heads * vdim for z and x, groups * N each for B
+    and C, one dt per head).  x | B | C pass a causal convolution with bias and SiLU (the
+    last taps - 1 inputs are per-sequence state); per head, with d = softplus(dt + dt_bias)
+    and a = exp(-exp(A_log) d):  S = a S + d B x^T,  y = S^T C + D x  (S [N, vdim], fp32,
+    per-sequence state); y * silu(z) is RMS-normed in ``inner_norm_groups`` parts, times a
+    weight (times ``out_scale``), and written into a column slice of the output
+    projection's input."""
+
+    def __init__(self, spec, eps: float, device, out_scale: float = 1.0):
+        super().__init__()
+        self.spec, self.eps, self.out_scale = spec, eps, float(out_scale)
+        H, P, N, G = spec.heads, spec.vdim, spec.dim, spec.kv_heads
+        assert H % G == 0 and (H * P) % spec.inner_norm_groups == 0
+        self.inner = H * P
+        self.n_conv = self.inner + 2 * G * N
+        self.n_in = self.inner + self.n_conv + H
+        self.n_out = self.inner
+        f = lambda *s: nn.Parameter(torch.zeros(*s, dtype=torch.float32, device=device),  # noqa: E731
+                                    requires_grad=False)
+        self.conv_w, self.conv_b = f(self.n_conv, spec.conv), f(self.n_conv)
+        self.dt_bias, self.a_log, self.dskip = f(H), f(H), f(H)
+        self.norm_weight = f(self.inner)         # the checkpoint's weight times out_scale
+
+    def state_shapes(self) -> tuple:
+        """Per-slot shapes: the convolution's last inputs, the recurrent state."""
+        sp = self.spec
+        return ((max(sp.conv - 1, 1), self.n_conv), (sp.heads, sp.dim, sp.vdim))
+
+    def forward(self, proj: torch.Tensor, col0: int, ctx: ForwardContext, state: tuple,
+                out: torch.Tensor) -> None:
+        sp = self.spec
+        z = proj[:, col0: col0 + self.inner]
+        xbc = ops.causal_conv(proj[:, col0 + self.inner: col0 + self.inner + self.n_conv],
+                              self.conv_w, self.conv_b, state[0], ctx.attn)
+        dt = proj[:, col0 + self.inner + self.n_conv: col0 + self.n_in]
+        y = ops.ssd_scan(xbc, dt, self.a_log, self.dt_bias, self.dskip, state[1], ctx.attn,
+                         sp.heads, sp.vdim, sp.dim, sp.kv_heads)
+        ops.gated_rms_norm(y, z, self.norm_weight, sp.inner_norm_groups, self.eps, True, out)
+
+
+class GatedDeltaCore(nn.Module):
+    """The gated delta rule mixer between its projections.  Its projection columns are
+    q | k (kv_heads * dim each) | v | output gate (heads * vdim each) | b | a (one per
+    head).  q | k | v pass a causal convolution without bias and SiLU; q and k become unit
+    vectors per head, q times dim^-1/2; with beta = sigmoid(b) and
+    g = exp(-exp(A_log) softplus(a + dt_bias)):  S = g S;  u = beta (v - S^T k);
+    S = S + k u^T;  o = S^T q  (S [dim, vdim], fp32, per-sequence state).  Each head's o
+    over its RMS, times a weight shared by the heads (times ``out_scale``), times
+    silu(output gate), into a column slice of the output projection's input."""
+
+    def __init__(self, spec, eps: float, device, out_scale: float = 1.0):
+        super().__init__()
+        self.spec, self.eps, self.out_scale = spec, eps, float(out_scale)
+        H, G, d, dv = spec.heads, spec.kv_heads, spec.dim, spec.vdim
+        assert H % G == 0
+        self.n_conv = 2 * G * d + H * dv
+        self.n_in = self.n_conv + H * dv + 2 * H
+        self.n_out = H * dv
+        f = lambda *s: nn.Parameter(torch.zeros(*s, dtype=torch.float32, device=device),  # noqa: E731
+                                    requires_grad=False)
+        self.conv_w = f(self.n_conv, spec.conv)
+        self.dt_bias, self.a_log = f(H), f(H)
+        self.norm_weight = f(H * dv)             # the shared weight per head, times out_scale
+
+    def state_shapes(self) -> tuple:
+        sp = self.spec
+        return ((max(sp.conv - 1, 1), self.n_conv), (sp.heads, sp.dim, sp.vdim))
+
+    def forward(self, proj: torch.Tensor, col0: int, ctx: ForwardContext, state: tuple,
+                out: torch.Tensor) -> None:
+        sp = self.spec
+        qkv = ops.causal_conv(proj[:, col0: col0 + self.n_conv], self.conv_w, None, state[0],
+                              ctx.attn)
+        g = proj[:, col0 + self.n_conv: col0 + self.n_conv + self.n_out]
+        ba = proj[:, col0 + self.n_conv + self.n_out: col0 + self.n_in]
+        o = ops.gated_delta_scan(qkv, ba, self.a_log, self.dt_bias, state[1], ctx.attn,
+                                 sp.heads, sp.kv_heads, sp.dim, sp.vdim)
+        ops.gated_rms_norm(o, g, self.norm_weight, sp.heads, self.eps, False, out)

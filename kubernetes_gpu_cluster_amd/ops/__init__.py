@@ -624,8 +624,8 @@ def fused_moe(x: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, topk_w: torc
 # results, xIELU, small fp32 gate projections, windowed attention with kept first tokens
 # over a plain-layout paged cache (per-layer query/key and value sizes), and the mLSTM
 # matrix-memory scan over per-sequence state slots.  ``meta`` is the step's AttnMetadata.
-GATE_SIGMOID, GATE_CAP_TANH, GATE_LOGSIG_CAP_TANH = (ref.GATE_SIGMOID, ref.GATE_CAP_TANH,
-                                                     ref.GATE_LOGSIG_CAP_TANH)
+GATE_SIGMOID, GATE_CAP_TANH, GATE_LOGSIG_CAP_TANH, GATE_NONE = (
+    ref.GATE_SIGMOID, ref.GATE_CAP_TANH, ref.GATE_LOGSIG_CAP_TANH, ref.GATE_NONE)
 
 
 def group_rms_norm(x: torch.Tensor, w: torch.Tensor, groups: int, eps: float,
@@ -682,12 +682,13 @@ def gate_proj(h: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], ki
 
 def rope_kv_store(qkv: torch.Tensor, positions: torch.Tensor, table: Optional[torch.Tensor],
                   k_cache: torch.Tensor, v_cache: torch.Tensor, slot_mapping: torch.Tensor,
-                  H: int, G: int, dk: int, dv: int) -> torch.Tensor:
+                  H: int, G: int, dk: int, dv: int, interleaved: bool = False) -> torch.Tensor:
     if not _gpu(qkv):
         return ref.rope_kv_store(qkv, positions, table, k_cache, v_cache, slot_mapping, H, G,
-                                 dk, dv)
+                                 dk, dv, interleaved)
     q = torch.empty(qkv.shape[0], H, dk, dtype=qkv.dtype, device=qkv.device)
-    _k().rope_kv_store(qkv, positions, table, q, k_cache, v_cache, slot_mapping, H, G, dk, dv)
+    _k().rope_kv_store(qkv, positions, table, q, k_cache, v_cache, slot_mapping, H, G, dk, dv,
+                       interleaved)
     return q
 
 
@@ -712,10 +713,13 @@ def window_attention_fast() -> bool:
 
 def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                      positions: torch.Tensor, meta, scale: float, window: int, keep_first: int,
-                     gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+                     gate: Optional[torch.Tensor] = None, softcap: float = 0.0,
+                     out_scale: float = 1.0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Prefill chunks and decode rows of one step alike: row t sees the cached keys
     j <= p with p - j < window or j < keep_first (p = positions[t]; window <= 0: plain
-    causal).  Decode padding rows (context length 0) give zeros."""
+    causal).  Decode padding rows (context length 0) give zeros.  ``softcap`` > 0: the
+    scaled scores pass softcap * tanh(. / softcap).  The result is multiplied by
+    ``out_scale`` and may go to ``out`` [T, H * dv], a column slice of a wider buffer."""
     T, H, _ = q.shape
     dv = v_cache.shape[3]
     if not _gpu(q):
@@ -723,9 +727,14 @@ def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
         if meta.num_decodes:
             tp = meta.num_prefill_tokens
             pos[tp:tp + meta.num_decodes] = meta.decode_ctx_lens[: meta.num_decodes].long() - 1
-        return ref.window_attention(q, k_cache, v_cache, pos, _row_tables(meta, T), scale,
-                                    window, keep_first, gate)
-    out = torch.empty(T, H * dv, dtype=q.dtype, device=q.device)
+        r = ref.window_attention(q, k_cache, v_cache, pos, _row_tables(meta, T), scale,
+                                 window, keep_first, gate, softcap, out_scale)
+        if out is not None:
+            out.copy_(r)
+            return out
+        return r
+    if out is None:
+        out = torch.empty(T, H * dv, dtype=q.dtype, device=q.device)
     ws, wb = getattr(meta, "work_seq", None), getattr(meta, "work_mblk", None)
     if meta.num_prefills and ws is None:
         qsl = meta.query_start_loc.tolist()
@@ -737,7 +746,8 @@ def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
                           meta.prefill_seq_lens, meta.prefill_block_tables,
                           meta.decode_ctx_lens, meta.decode_block_tables, ws, wb,
                           meta.num_prefills, meta.num_decodes, meta.num_prefill_tokens,
-                          scale, window, keep_first, gate, window_attention_fast())
+                          scale, window, keep_first, gate, window_attention_fast(),
+                          float(softcap), float(out_scale))
     return out
 
 
@@ -852,13 +862,20 @@ def latent_rope_store(proj: torch.Tensor, q_lat: torch.Tensor, positions: torch.
     return q
 
 
-def gate_mul(o: torch.Tensor, g: torch.Tensor) -> torch.Tensor:
-    """o [T, H, dv] (any token / head strides) * sigmoid(g [T, H dv], a column slice)."""
+def gate_mul(o: torch.Tensor, g: torch.Tensor, scale: float = 1.0,
+             out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """o [T, H, dv] (any token / head strides) * sigmoid(g [T, H dv], a column slice) *
+    scale, into ``out`` [T, H dv] (a column slice of a wider buffer) when given."""
     if not _gpu(o):
-        return ref.gate_mul(o, g)
+        r = ref.gate_mul(o, g, scale)
+        if out is not None:
+            out.copy_(r)
+            return out
+        return r
     T, H, dv = o.shape
-    out = torch.empty(T, H * dv, dtype=g.dtype, device=g.device)
-    _k().gate_mul(out, o, g)
+    if out is None:
+        out = torch.empty(T, H * dv, dtype=g.dtype, device=g.device)
+    _k().gate_mul(out, o, g, float(scale))
     return out
 
 
@@ -956,3 +973,68 @@ def side_input(x: torch.Tensor, y: Optional[torch.Tensor], mult: float, gate_w: 
     if next_w is None:
         out_dtype = None
     return residual_norm(x, linear(g, proj_w), mult, next_w, eps, out_dtype, add_norm_w=side_w)
+
+
+# ------------------------------------------------------------------ parallel mixers
+# An attention and a recurrence side by side on one input: short causal convolutions over
+# per-sequence state, the Mamba-2 recurrence, the gated delta rule, and RMS norms combined
+# with a SiLU gate.  State tensors hold one fp32 entry per sequence slot; a chunk that
+# starts at position 0 starts from zeros, and rows of slot < 0 (graph padding) are skipped.
+def causal_conv(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor],
+                state: torch.Tensor, meta, silu: bool = True) -> torch.Tensor:
+    """fp32 [T, C]: y[t, c] = act(sum_j w[c, j] x[t - (K - 1) + j, c] + bias[c]) per
+    sequence; x [T, C] is a column slice of a projection, w fp32 [C, K], state fp32
+    [slots, K - 1, C] each sequence's last K - 1 inputs (read, then replaced)."""
+    if not _gpu(x):
+        return ref.causal_conv(x, w, bias, state, ref.step_sequences(meta), silu)
+    out = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+    _k().causal_conv(out, x, w, bias, state, meta.query_start_loc, meta.prefill_seq_lens,
+                     meta.decode_ctx_lens, meta.state_slots, meta.num_prefills,
+                     meta.num_decodes, meta.num_prefill_tokens, silu)
+    return out
+
+
+def ssd_scan(xbc: torch.Tensor, dt: torch.Tensor, a_log: torch.Tensor, dt_bias: torch.Tensor,
+             dskip: torch.Tensor, state: torch.Tensor, meta, H: int, P: int, N: int,
+             G: int) -> torch.Tensor:
+    """fp32 [T, H P]: the Mamba-2 recurrence over every step sequence's rows from / into
+    state [slots, H, N, P]; xbc fp32 [T, H P + 2 G N] = x | B | C, dt [T, H] (a column
+    slice of the projection); see ``ref.ssd_scan``."""
+    if not _gpu(xbc):
+        return ref.ssd_scan(xbc, dt, a_log, dt_bias, dskip, state, ref.step_sequences(meta),
+                            H, P, N, G)
+    out = torch.empty(xbc.shape[0], H * P, dtype=torch.float32, device=xbc.device)
+    _k().ssd_scan(out, xbc, dt, a_log, dt_bias, dskip, state, meta.query_start_loc,
+                  meta.prefill_seq_lens, meta.decode_ctx_lens, meta.state_slots,
+                  meta.num_prefills, meta.num_decodes, meta.num_prefill_tokens, H, P, N, G)
+    return out
+
+
+def gated_delta_scan(qkv: torch.Tensor, ba: torch.Tensor, a_log: torch.Tensor,
+                     dt_bias: torch.Tensor, state: torch.Tensor, meta, H: int, G: int, d: int,
+                     dv: int) -> torch.Tensor:
+    """fp32 [T, H dv]: the gated delta rule over every step sequence's rows from / into
+    state [slots, H, d, dv]; qkv fp32 [T, 2 G d + H dv] = q | k | v, ba [T, 2 H] (a column
+    slice of the projection) = write strength | decay pre-activations; see
+    ``ref.gated_delta_scan``."""
+    if not _gpu(qkv):
+        return ref.gated_delta_scan(qkv, ba, a_log, dt_bias, state, ref.step_sequences(meta),
+                                    H, G, d, dv)
+    out = torch.empty(qkv.shape[0], H * dv, dtype=torch.float32, device=qkv.device)
+    _k().gated_delta_scan(out, qkv, ba, a_log, dt_bias, state, meta.query_start_loc,
+                          meta.prefill_seq_lens, meta.decode_ctx_lens, meta.state_slots,
+                          meta.num_prefills, meta.num_decodes, meta.num_prefill_tokens, H, G,
+                          d, dv)
+    return out
+
+
+def gated_rms_norm(y: torch.Tensor, gate: torch.Tensor, w: torch.Tensor, groups: int,
+                   eps: float, gate_first: bool, out: torch.Tensor) -> torch.Tensor:
+    """out [T, n] (a column slice of a wider buffer) = RMS norm of y (fp32 [T, n]) in
+    ``groups`` parts, times w, with silu(gate [T, n], a column slice) applied before the
+    norm (gate_first) or after it."""
+    if not _gpu(y):
+        out.copy_(ref.gated_rms_norm(y, gate, w, groups, eps, gate_first, out.dtype))
+        return out
+    _k().gated_rms_norm(out, y, gate, w, groups, eps, gate_first)
+    return out

@@ -386,12 +386,14 @@ def xielu(z: torch.Tensor, ab: torch.Tensor) -> torch.Tensor:
                        b * (torch.expm1(torch.clamp(zf, max=0.0)) - zf) + 0.5 * zf).to(z.dtype)
 
 
-GATE_SIGMOID, GATE_CAP_TANH, GATE_LOGSIG_CAP_TANH = 0, 1, 2
+GATE_SIGMOID, GATE_CAP_TANH, GATE_LOGSIG_CAP_TANH, GATE_NONE = 0, 1, 2, 3
 
 
 def _gate_act(y: torch.Tensor, kind: int, cap: float) -> torch.Tensor:
     if kind == GATE_SIGMOID:
         return torch.sigmoid(y)
+    if kind == GATE_NONE:
+        return y
     y = cap * torch.tanh(y / cap)
     return y if kind == GATE_CAP_TANH else torch.nn.functional.logsigmoid(y)
 
@@ -418,11 +420,12 @@ def rope_table(rot_dims: int, max_pos: int, base: float) -> torch.Tensor:
 
 def rope_kv_store(qkv: torch.Tensor, positions: torch.Tensor, table: Optional[torch.Tensor],
                   k_cache: torch.Tensor, v_cache: torch.Tensor, slot_mapping: torch.Tensor,
-                  H: int, G: int, dk: int, dv: int) -> torch.Tensor:
+                  H: int, G: int, dk: int, dv: int, interleaved: bool = False) -> torch.Tensor:
     """qkv [T, H*dk + G*dk + G*dv] -> rotated q [T, H, dk]; rotated k and v go to the
     plain-layout paged cache (k_cache [nb, G, bs, dk], v_cache [nb, G, bs, dv]) at
-    ``slot_mapping`` (< 0: no write).  Rotation pairs dim i with i + rot/2 over the first
-    rot = table.shape[1] dims of a head (fp32 math); the rest pass unchanged."""
+    ``slot_mapping`` (< 0: no write).  Rotation pairs dim i with i + rot/2 (interleaved:
+    2i with 2i + 1) over the first rot = table.shape[1] dims of a head (fp32 math); the
+    rest pass unchanged."""
     T = qkv.shape[0]
     q = qkv[:, : H * dk].float().view(T, H, dk)
     k = qkv[:, H * dk: (H + G) * dk].float().view(T, G, dk)
@@ -433,6 +436,10 @@ def rope_kv_store(qkv: torch.Tensor, positions: torch.Tensor, table: Optional[to
         c, s = cs[:, None, : r // 2], cs[:, None, r // 2:]
 
         def rot(x):
+            if interleaved:
+                a, b = x[..., 0:r:2], x[..., 1:r:2]
+                ab = torch.stack([a * c - b * s, b * c + a * s], dim=-1).flatten(-2)
+                return torch.cat([ab, x[..., r:]], dim=-1)
             a, b = x[..., : r // 2], x[..., r // 2: r]
             return torch.cat([a * c - b * s, b * c + a * s, x[..., r:]], dim=-1)
         q, k = rot(q), rot(k)
@@ -447,12 +454,14 @@ def rope_kv_store(qkv: torch.Tensor, positions: torch.Tensor, table: Optional[to
 def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                      positions: torch.Tensor, row_tables: torch.Tensor, scale: float,
                      window: int, keep_first: int,
-                     gate: Optional[torch.Tensor]) -> torch.Tensor:
+                     gate: Optional[torch.Tensor], softcap: float = 0.0,
+                     out_scale: float = 1.0) -> torch.Tensor:
     """q [T, H, dk] (rotated; the step's k / v already stored) -> [T, H*dv].  Row t at
     position p = positions[t] attends the cached keys j <= p with p - j < window or
     j < keep_first (window <= 0: all of them) of the sequence whose block table is
-    row_tables[t]; softmax and the weighted sum in fp32; each head's output times
-    gate[t, head] (fp32) when given."""
+    row_tables[t]; scores q.k * scale, then softcap * tanh(score / softcap) when
+    softcap > 0; softmax and the weighted sum in fp32; each head's output times
+    gate[t, head] (fp32) when given, and times out_scale."""
     T, H, dk = q.shape
     G, bs, dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[3]
     out = torch.zeros(T, H, dv, dtype=torch.float32)
@@ -468,10 +477,14 @@ def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
         v = v_cache[blk, :, j % bs].float()
         qt = q[t].float().view(G, H // G, dk)
         s = torch.einsum("ghd,ngd->ghn", qt, k) * scale
+        if softcap > 0:
+            s = softcap * torch.tanh(s / softcap)
         pr = torch.softmax(s, dim=-1)
         out[t] = torch.einsum("ghn,ngv->ghv", pr, v).reshape(H, dv)
     if gate is not None:
         out = out * gate.float()[:, :, None]
+    if out_scale != 1.0:
+        out = out * out_scale
     return out.view(T, H * dv).to(q.dtype)
 
 
@@ -659,10 +672,11 @@ def latent_rope_store(proj: torch.Tensor, q_lat: torch.Tensor, positions: torch.
     return torch.cat([q_lat.float().transpose(0, 1), q], -1).to(proj.dtype)
 
 
-def gate_mul(o: torch.Tensor, g: torch.Tensor) -> torch.Tensor:
-    """o [T, H, dv] (any strides) * sigmoid(g [T, H dv]) -> [T, H dv] in g's dtype."""
+def gate_mul(o: torch.Tensor, g: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+    """o [T, H, dv] (any strides) * sigmoid(g [T, H dv]) * scale -> [T, H dv] in g's dtype."""
     T = o.shape[0]
-    return (o.float().reshape(T, -1) * torch.sigmoid(g.float())).to(g.dtype)
+    y = o.float().reshape(T, -1) * torch.sigmoid(g.float())
+    return (y * scale if scale != 1.0 else y).to(g.dtype)
 
 
 def relu_sq(z: torch.Tensor) -> torch.Tensor:
@@ -703,3 +717,105 @@ def side_gate(pre: torch.Tensor, ids: torch.Tensor, table: torch.Tensor, col0: i
     z = pre.float()
     g = 0.5 * z * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z ** 3)))
     return (g * table[ids.long(), col0:col0 + n].float()).to(pre.dtype)
+
+
+# ---------------------------------------------------------------- parallel mixers
+# (short causal convolutions over per-sequence state, the Mamba-2 recurrence, the gated
+# delta rule, RMS norms combined with a SiLU gate)
+def causal_conv(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor],
+                state: torch.Tensor, seqs: list, silu: bool = True) -> torch.Tensor:
+    """Per-channel causal convolution over time: y[t, c] = sum_j w[c, j] * x[t - (K-1) + j, c]
+    (+ bias[c]), the last tap on the current token, then SiLU.  x [T, C] (a column slice of
+    a projection), w fp32 [C, K].  state fp32 [slots, K-1, C] holds each sequence's last
+    K-1 inputs (oldest first; zeros before position 0) and is updated.  -> fp32 [T, C]."""
+    T, C = x.shape
+    K = w.shape[1]
+    out = torch.zeros(T, C, dtype=torch.float32, device=x.device)
+    wf = w.float()
+    for a, n, p0, slot in seqs:
+        if slot < 0:
+            continue
+        prev = torch.zeros(K - 1, C) if p0 == 0 else state[slot].clone()
+        xs = torch.cat([prev, x[a:a + n].float()], 0)              # [K-1+n, C]
+        y = torch.zeros(n, C)
+        for j in range(K):
+            y = y + xs[j:j + n] * wf[:, j]
+        if bias is not None:
+            y = y + bias.float()
+        out[a:a + n] = y
+        if K > 1:
+            state[slot] = xs[n:]
+    return out * torch.sigmoid(out) if silu else out
+
+
+def ssd_scan(xbc: torch.Tensor, dt: torch.Tensor, a_log: torch.Tensor, dt_bias: torch.Tensor,
+             dskip: torch.Tensor, state: torch.Tensor, seqs: list, H: int, P: int, N: int,
+             G: int) -> torch.Tensor:
+    """The Mamba-2 recurrence.  xbc fp32 [T, H P + 2 G N] = x | B | C (after convolution
+    and SiLU), dt [T, H] raw step sizes; per head h (group g = h // (H / G)):
+        d = softplus(dt + dt_bias_h);  S = exp(-exp(a_log_h) d) S + d B_g x_h^T  (S [N, P])
+        y_h = S^T C_g + dskip_h x_h
+    from state[slot] [H, N, P] fp32 (zeros at position 0), written back.  -> fp32 [T, H P]."""
+    T = xbc.shape[0]
+    x = xbc[:, : H * P].float().view(T, H, P)
+    B = xbc[:, H * P: H * P + G * N].float().view(T, G, N).repeat_interleave(H // G, dim=1)
+    C = xbc[:, H * P + G * N: H * P + 2 * G * N].float().view(T, G, N).repeat_interleave(H // G, dim=1)
+    d = torch.nn.functional.softplus(dt.float() + dt_bias.float())
+    decay = torch.exp(-torch.exp(a_log.float()) * d)
+    out = torch.zeros(T, H, P, dtype=torch.float32)
+    for a, n, p0, slot in seqs:
+        if slot < 0:
+            continue
+        S = torch.zeros(H, N, P) if p0 == 0 else state[slot].clone()
+        for t in range(a, a + n):
+            S = decay[t, :, None, None] * S + (d[t, :, None] * B[t])[:, :, None] * x[t][:, None, :]
+            out[t] = torch.einsum("hnp,hn->hp", S, C[t]) + dskip.float()[:, None] * x[t]
+        state[slot] = S
+    return out.view(T, H * P)
+
+
+def gated_delta_scan(qkv: torch.Tensor, ba: torch.Tensor, a_log: torch.Tensor,
+                     dt_bias: torch.Tensor, state: torch.Tensor, seqs: list, H: int, G: int,
+                     d: int, dv: int) -> torch.Tensor:
+    """The gated delta rule.  qkv fp32 [T, 2 G d + H dv] = q | k | v (after convolution and
+    SiLU), ba [T, 2 H]: pre-activations of the write strength | of the decay.  q and k
+    become unit vectors per head (x / sqrt(sum x^2 + 1e-6)), q times d^-1/2.  Per head h
+    (q / k head h // (H / G)), with beta = sigmoid(b), g = exp(-exp(a_log_h) softplus(a + dt_bias_h)):
+        S = g S;  u = beta (v - S^T k);  S = S + k u^T;  o = S^T q         (S [d, dv])
+    from state[slot] [H, d, dv] fp32 (zeros at position 0), written back.  -> fp32 [T, H dv]."""
+    T = qkv.shape[0]
+    q = qkv[:, : G * d].float().view(T, G, d)
+    k = qkv[:, G * d: 2 * G * d].float().view(T, G, d)
+    v = qkv[:, 2 * G * d: 2 * G * d + H * dv].float().view(T, H, dv)
+    q = q * torch.rsqrt(q.pow(2).sum(-1, keepdim=True) + 1e-6) * d ** -0.5
+    k = k * torch.rsqrt(k.pow(2).sum(-1, keepdim=True) + 1e-6)
+    q, k = q.repeat_interleave(H // G, dim=1), k.repeat_interleave(H // G, dim=1)
+    beta = torch.sigmoid(ba[:, :H].float())
+    g = torch.exp(-torch.exp(a_log.float()) *
+                  torch.nn.functional.softplus(ba[:, H: 2 * H].float() + dt_bias.float()))
+    out = torch.zeros(T, H, dv, dtype=torch.float32)
+    for a, n, p0, slot in seqs:
+        if slot < 0:
+            continue
+        S = torch.zeros(H, d, dv) if p0 == 0 else state[slot].clone()
+        for t in range(a, a + n):
+            S = g[t, :, None, None] * S
+            u = beta[t, :, None] * (v[t] - torch.einsum("hdv,hd->hv", S, k[t]))
+            S = S + k[t][:, :, None] * u[:, None, :]
+            out[t] = torch.einsum("hdv,hd->hv", S, q[t])
+        state[slot] = S
+    return out.view(T, H * dv)
+
+
+def gated_rms_norm(y: torch.Tensor, gate: torch.Tensor, w: torch.Tensor, groups: int,
+                   eps: float, gate_first: bool, out_dtype: torch.dtype) -> torch.Tensor:
+    """y fp32 [T, n] in ``groups`` equal parts, each divided by its own root mean square and
+    the row multiplied by w [n], with a SiLU gate silu(gate [T, n]): applied to y before
+    the norm (gate_first) or to the normed, weighted result.  fp32 math -> out_dtype."""
+    T, n = y.shape
+    g = gate.float()
+    g = g * torch.sigmoid(g)
+    v = y.float() * g if gate_first else y.float()
+    vg = v.view(T, groups, n // groups)
+    v = (vg * torch.rsqrt(vg.pow(2).mean(-1, keepdim=True) + eps)).view(T, n) * w.float()
+    return (v if gate_first else v * g).to(out_dtype)
