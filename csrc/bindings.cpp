@@ -1307,7 +1307,7 @@ void gate_proj(Tensor out, Tensor h, Tensor w, std::optional<Tensor> bias, int64
   const int64_t W = h.size(1), N = w.size(0);
   TORCH_CHECK(W * 4 <= 64 * 1024, "kgc.gate_proj: W <= 16384");
   TORCH_CHECK(out.dim() == 2 && out.size(0) == h.size(0) && out.size(1) == N, "kgc.gate_proj: out");
-  TORCH_CHECK(kind_a >= 0 && kind_a <= 2 && kind_b >= 0 && kind_b <= 2 && cap > 0, "kinds / cap");
+  TORCH_CHECK(kind_a >= 0 && kind_a <= 3 && kind_b >= 0 && kind_b <= 3 && cap > 0, "kinds / cap");
   const float* bp = nullptr;
   if (bias.has_value()) {
     check_f32(*bias, "bias");
@@ -1333,7 +1333,7 @@ void check_plain_cache(const Tensor& kc, const Tensor& vc, const Tensor& like, i
 
 void rope_kv_store(Tensor qkv, Tensor positions, std::optional<Tensor> table, Tensor q_out,
                    Tensor k_cache, Tensor v_cache, Tensor slots, int64_t H, int64_t G, int64_t dk,
-                   int64_t dv) {
+                   int64_t dv, bool interleaved) {
   check_gpu(qkv, "qkv");
   c10::hip::HIPGuardMasqueradingAsCUDA g(qkv.device());
   TORCH_CHECK(qkv.dim() == 2 && qkv.stride(1) == 1 && act_dtype(qkv) &&
@@ -1360,7 +1360,7 @@ void rope_kv_store(Tensor qkv, Tensor positions, std::optional<Tensor> table, Te
                             positions.data_ptr<int64_t>(), tp, (int)rot, (int)rows,
                             q_out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                             slots.data_ptr<int64_t>(), (int)T, (int)H, (int)G, (int)dk, (int)dv,
-                            (int)k_cache.size(2), (int)k_cache.size(0), stream());
+                            (int)k_cache.size(2), (int)k_cache.size(0), interleaved, stream());
 }
 
 const int* i32_ptr(const std::optional<Tensor>& t, int64_t min_numel, const char* name) {
@@ -1386,7 +1386,7 @@ void window_attention(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
                       std::optional<Tensor> dbt, std::optional<Tensor> work_seq,
                       std::optional<Tensor> work_blk, int64_t P, int64_t D, int64_t Tp,
                       double scale, int64_t window, int64_t keep_first,
-                      std::optional<Tensor> gate, bool fast) {
+                      std::optional<Tensor> gate, bool fast, double softcap, double out_scale) {
   check_gpu(q, "q");
   c10::hip::HIPGuardMasqueradingAsCUDA g(q.device());
   TORCH_CHECK(q.dim() == 3 && q.is_contiguous() && act_dtype(q), "kgc.window_attention: q [T, H, dk]");
@@ -1416,8 +1416,14 @@ void window_attention(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
                        reinterpret_cast<uintptr_t>(v_cache.data_ptr()) % 16 == 0;
   TORCH_CHECK(G >= 1 && H % G == 0 && H <= 65535, "kgc.window_attention: heads");
   TORCH_CHECK(dk <= 4096 && dv <= kgc::window_attention_max_dv(), "kgc.window_attention: head sizes");
-  TORCH_CHECK(out.is_contiguous() && out.numel() == T * H * dv &&
-              out.scalar_type() == q.scalar_type(), "kgc.window_attention: out [T, H * dv]");
+  TORCH_CHECK(out.is_cuda() && out.device() == q.device() && out.dim() == 2 && out.size(0) == T &&
+              out.size(1) == H * dv && out.stride(1) == 1 && (T <= 1 || out.stride(0) >= H * dv) &&
+              out.scalar_type() == q.scalar_type(),
+              "kgc.window_attention: out [T, H * dv] (rows may be slices of a wider buffer)");
+  const kgc::WindowExtra ex{T > 1 ? out.stride(0) : H * dv, (float)softcap, (float)out_scale};
+  // the matrix-core kernel stores 8-byte pieces of a row
+  const bool out_vec = reinterpret_cast<uintptr_t>(out.data_ptr()) % 8 == 0 &&
+                       ex.ors * out.element_size() % 8 == 0;
   TORCH_CHECK(P >= 0 && D >= 0 && Tp >= 0 && (P > 0) == (Tp > 0) && Tp + D == T,
               "kgc.window_attention: T must be prefill tokens + decode rows");
   const int64_t bts = table_stride(pbt, P, table_stride(dbt, D, 0));
@@ -1435,7 +1441,7 @@ void window_attention(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
   const int* dp = i32_ptr(dbt, D, "decode block tables");
   const int bs = (int)k_cache.size(2), nb = (int)k_cache.size(0), dt = dt_code(q);
   int rest = 3;                   // row kinds the one-wave kernel still has to run
-  if (fast && aligned && P > 0 && work_seq.has_value() && work_blk.has_value() &&
+  if (fast && aligned && out_vec && P > 0 && work_seq.has_value() && work_blk.has_value() &&
       kgc::window_prefill_mfma_ok(dt, (int)dk, (int)dv)) {
     const int64_t nw = work_seq->numel();
     TORCH_CHECK(work_blk->numel() == nw && work_seq->scalar_type() == at::kInt &&
@@ -1445,7 +1451,8 @@ void window_attention(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
                                     v_cache.data_ptr(), qp, sp, pp, (int)bts,
                                     work_seq->data_ptr<int>(), work_blk->data_ptr<int>(), (int)nw,
                                     kgc::prefill_block_m(), (int)H, (int)G, (int)dk, (int)dv,
-                                    (int)krs, (int)vrs, bs, nb, (float)scale, (int)window, (int)keep_first, gp, stream());
+                                    (int)krs, (int)vrs, bs, nb, (float)scale, (int)window, (int)keep_first, gp, ex,
+                                    stream());
     rest &= ~1;
   }
   if (fast && aligned && D > 0 && kgc::window_decode_ok((int)dk, (int)dv, (int)(H / G)) &&
@@ -1453,7 +1460,7 @@ void window_attention(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
     kgc::launch_window_decode(dt, out.data_ptr(), q.data_ptr(), k_cache.data_ptr(),
                               v_cache.data_ptr(), cp, dp, (int)bts, (int)Tp, (int)D, (int)H,
                               (int)G, (int)dk, (int)dv, (int)krs, (int)vrs, bs, nb, (float)scale,
-                              (int)window, (int)keep_first, gp, stream());
+                              (int)window, (int)keep_first, gp, ex, stream());
     rest &= ~2;
   }
   if (!P) rest &= ~1;
@@ -1461,7 +1468,7 @@ void window_attention(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
   kgc::launch_window_attention(dt, out.data_ptr(), q.data_ptr(), k_cache.data_ptr(),
                                v_cache.data_ptr(), qp, sp, pp, cp, dp, (int)bts, (int)P, (int)Tp,
                                (int)T, (int)H, (int)G, (int)dk, (int)dv, (int)krs, (int)vrs, bs, nb,
-                               (float)scale, (int)window, (int)keep_first, gp, rest, stream());
+                               (float)scale, (int)window, (int)keep_first, gp, rest, ex, stream());
 }
 
 void mlstm_scan(Tensor out, Tensor qkvg, Tensor gates, Tensor S, Tensor n, Tensor m,
@@ -1499,6 +1506,130 @@ const float* f32_opt(const std::optional<Tensor>& t, int64_t numel, const char* 
   check_f32(*t, name);
   TORCH_CHECK(t->numel() == numel, "kgc: ", name, " must have ", numel, " entries");
   return t->data_ptr<float>();
+}
+
+// ---- parallel mixers: convolution state, Mamba-2, gated delta rule, gated RMS norm ----------
+void check_step(const char* op, int64_t T, int64_t P, int64_t D, int64_t Tp) {
+  TORCH_CHECK(Tp + D == T && P >= 0 && D >= 0 && (P > 0) == (Tp > 0), "kgc.", op, ": step counts");
+}
+
+// a [T, n] column slice of a wider activation matrix
+void check_cols(const Tensor& t, int64_t T, int64_t n, const Tensor& like, const char* name) {
+  TORCH_CHECK(t.is_cuda() && t.device() == like.device() && t.dim() == 2 && t.size(0) == T &&
+              t.size(1) == n && t.stride(1) == 1 && act_dtype(t), "kgc: ", name, " [T, ", n,
+              "] (a column slice)");
+}
+
+void causal_conv(Tensor out, Tensor x, Tensor w, std::optional<Tensor> bias, Tensor state,
+                 std::optional<Tensor> qsl, std::optional<Tensor> seq_lens,
+                 std::optional<Tensor> ctx_lens, Tensor slots, std::optional<Tensor> work_seq,
+                 std::optional<Tensor> work_blk, int64_t P, int64_t D, int64_t Tp, bool silu) {
+  check_gpu(x, "x");
+  check_f32(out, "out");
+  check_f32(w, "w");
+  check_f32(state, "state");
+  c10::hip::HIPGuardMasqueradingAsCUDA g(x.device());
+  TORCH_CHECK(x.dim() == 2, "kgc.causal_conv: x [T, C]");
+  const int64_t T = x.size(0), C = x.size(1);
+  check_cols(x, T, C, x, "x");
+  check_step("causal_conv", T, P, D, Tp);
+  TORCH_CHECK(w.dim() == 2 && w.size(0) == C && w.is_contiguous() && w.size(1) >= 1 &&
+              w.size(1) <= kgc::causal_conv_max_taps(), "kgc.causal_conv: w [C, taps <= 8]");
+  const int64_t K = w.size(1);
+  TORCH_CHECK(out.is_contiguous() && out.numel() == T * C, "kgc.causal_conv: out [T, C]");
+  TORCH_CHECK(state.is_contiguous() && state.dim() == 3 && state.size(2) == C &&
+              (K == 1 || state.size(1) == K - 1), "kgc.causal_conv: state [slots, taps - 1, C]");
+  int64_t nw = 0;
+  const int* wsp = nullptr;
+  const int* wbp = nullptr;
+  if (P > 0) {
+    TORCH_CHECK(work_seq.has_value() && work_blk.has_value() && work_seq->is_cuda() &&
+                work_blk->is_cuda() && work_seq->scalar_type() == at::kInt &&
+                work_blk->scalar_type() == at::kInt && work_seq->numel() == work_blk->numel(),
+                "kgc.causal_conv: work list int32 [n] on the GPU");
+    nw = work_seq->numel();
+    wsp = work_seq->data_ptr<int>();
+    wbp = work_blk->data_ptr<int>();
+  }
+  kgc::launch_causal_conv(dt_code(x), out.data_ptr<float>(), x.data_ptr(), x.stride(0),
+                          w.data_ptr<float>(), f32_opt(bias, C, "bias"), state.data_ptr<float>(),
+                          i32_ptr(qsl, P ? P + 1 : 0, "query_start_loc"),
+                          i32_ptr(seq_lens, P, "seq_lens"), i32_ptr(ctx_lens, D, "ctx_lens"),
+                          i32_ptr(slots, P + D, "state slots"), wsp, wbp, (int)nw,
+                          kgc::prefill_block_m(), (int)P, (int)D, (int)Tp, (int)C, (int)K,
+                          (int)state.size(0), silu, stream());
+}
+
+void ssd_scan(Tensor out, Tensor xbc, Tensor dt, Tensor a_log, Tensor dt_bias, Tensor dskip,
+              Tensor S, std::optional<Tensor> qsl, std::optional<Tensor> seq_lens,
+              std::optional<Tensor> ctx_lens, Tensor slots, int64_t P, int64_t D, int64_t Tp,
+              int64_t H, int64_t V, int64_t N, int64_t G) {
+  check_gpu(xbc, "xbc");
+  check_f32(out, "out");
+  check_f32(xbc, "xbc");
+  check_f32(S, "S");
+  c10::hip::HIPGuardMasqueradingAsCUDA g(xbc.device());
+  TORCH_CHECK(H >= 1 && H <= 65535 && G >= 1 && H % G == 0 && V >= 1 && N >= 1 &&
+              N <= kgc::matrix_scan_max_rows(), "kgc.ssd_scan: head sizes");
+  TORCH_CHECK(xbc.dim() == 2 && xbc.is_contiguous() && xbc.size(1) == H * V + 2 * G * N,
+              "kgc.ssd_scan: xbc [T, H V + 2 G N]");
+  const int64_t T = xbc.size(0);
+  check_step("ssd_scan", T, P, D, Tp);
+  check_cols(dt, T, H, xbc, "dt");
+  TORCH_CHECK(out.is_contiguous() && out.numel() == T * H * V, "kgc.ssd_scan: out [T, H V]");
+  TORCH_CHECK(S.is_contiguous() && S.dim() == 4 && S.size(1) == H && S.size(2) == N &&
+              S.size(3) == V, "kgc.ssd_scan: state [slots, H, N, V]");
+  kgc::launch_ssd_scan(dt_code(dt), out.data_ptr<float>(), xbc.data_ptr<float>(), dt.data_ptr(),
+                       dt.stride(0), f32_opt(a_log, H, "a_log"), f32_opt(dt_bias, H, "dt_bias"),
+                       f32_opt(dskip, H, "dskip"), S.data_ptr<float>(),
+                       i32_ptr(qsl, P ? P + 1 : 0, "query_start_loc"),
+                       i32_ptr(seq_lens, P, "seq_lens"), i32_ptr(ctx_lens, D, "ctx_lens"),
+                       i32_ptr(slots, P + D, "state slots"), (int)P, (int)D, (int)Tp, (int)H,
+                       (int)V, (int)N, (int)G, (int)S.size(0), stream());
+}
+
+void gated_delta_scan(Tensor out, Tensor qkv, Tensor ba, Tensor a_log, Tensor dt_bias, Tensor S,
+                      std::optional<Tensor> qsl, std::optional<Tensor> seq_lens,
+                      std::optional<Tensor> ctx_lens, Tensor slots, int64_t P, int64_t D,
+                      int64_t Tp, int64_t H, int64_t G, int64_t d, int64_t V) {
+  check_gpu(qkv, "qkv");
+  check_f32(out, "out");
+  check_f32(qkv, "qkv");
+  check_f32(S, "S");
+  c10::hip::HIPGuardMasqueradingAsCUDA g(qkv.device());
+  TORCH_CHECK(H >= 1 && H <= 65535 && G >= 1 && H % G == 0 && V >= 1 && d >= 1 &&
+              d <= kgc::matrix_scan_max_rows(), "kgc.gated_delta_scan: head sizes");
+  TORCH_CHECK(qkv.dim() == 2 && qkv.is_contiguous() && qkv.size(1) == 2 * G * d + H * V,
+              "kgc.gated_delta_scan: qkv [T, 2 G d + H V]");
+  const int64_t T = qkv.size(0);
+  check_step("gated_delta_scan", T, P, D, Tp);
+  check_cols(ba, T, 2 * H, qkv, "ba");
+  TORCH_CHECK(out.is_contiguous() && out.numel() == T * H * V, "kgc.gated_delta_scan: out [T, H V]");
+  TORCH_CHECK(S.is_contiguous() && S.dim() == 4 && S.size(1) == H && S.size(2) == d &&
+              S.size(3) == V, "kgc.gated_delta_scan: state [slots, H, d, V]");
+  kgc::launch_gated_delta_scan(dt_code(ba), out.data_ptr<float>(), qkv.data_ptr<float>(),
+                               ba.data_ptr(), ba.stride(0), f32_opt(a_log, H, "a_log"),
+                               f32_opt(dt_bias, H, "dt_bias"), S.data_ptr<float>(),
+                               i32_ptr(qsl, P ? P + 1 : 0, "query_start_loc"),
+                               i32_ptr(seq_lens, P, "seq_lens"), i32_ptr(ctx_lens, D, "ctx_lens"),
+                               i32_ptr(slots, P + D, "state slots"), (int)P, (int)D, (int)Tp,
+                               (int)H, (int)G, (int)d, (int)V, (int)S.size(0), stream());
+}
+
+void gated_rms_norm(Tensor out, Tensor y, Tensor gate, Tensor w, int64_t groups, double eps,
+                    bool gate_first) {
+  check_gpu(y, "y");
+  check_f32(y, "y");
+  c10::hip::HIPGuardMasqueradingAsCUDA g(y.device());
+  TORCH_CHECK(y.dim() == 2 && y.is_contiguous(), "kgc.gated_rms_norm: y [T, n]");
+  const int64_t T = y.size(0), n = y.size(1);
+  TORCH_CHECK(groups >= 1 && n % groups == 0, "kgc.gated_rms_norm: parts");
+  check_cols(gate, T, n, y, "gate");
+  check_cols(out, T, n, y, "out");
+  TORCH_CHECK(out.scalar_type() == gate.scalar_type(), "kgc.gated_rms_norm: out / gate dtypes");
+  kgc::launch_gated_rms_norm(dt_code(gate), out.data_ptr(), out.stride(0), y.data_ptr<float>(),
+                             gate.data_ptr(), gate.stride(0), f32_opt(w, n, "w"), (int)T, (int)n,
+                             (int)groups, (float)eps, gate_first, stream());
 }
 
 void residual_norm(std::optional<Tensor> out, Tensor x, std::optional<Tensor> add,
@@ -1628,7 +1759,7 @@ void latent_rope_store(Tensor q_out, Tensor proj, Tensor q_lat, Tensor positions
                                 (int)H, (int)d, (int)r, (int)rank, stream());
 }
 
-void gate_mul(Tensor out, Tensor o, Tensor gt) {
+void gate_mul(Tensor out, Tensor o, Tensor gt, double scale) {
   check_gpu(o, "o");
   c10::hip::HIPGuardMasqueradingAsCUDA g(o.device());
   TORCH_CHECK(o.dim() == 3 && o.stride(2) == 1 && act_dtype(o), "kgc.gate_mul: o [T, H, dv]");
@@ -1636,10 +1767,12 @@ void gate_mul(Tensor out, Tensor o, Tensor gt) {
   TORCH_CHECK(gt.is_cuda() && gt.dim() == 2 && gt.size(0) == T && gt.size(1) == H * dv &&
               gt.stride(1) == 1 && gt.scalar_type() == o.scalar_type() && gt.device() == o.device(),
               "kgc.gate_mul: gate [T, H dv]");
-  TORCH_CHECK(out.is_cuda() && out.is_contiguous() && out.numel() == T * H * dv &&
+  TORCH_CHECK(out.is_cuda() && out.dim() == 2 && out.size(0) == T && out.size(1) == H * dv &&
+              out.stride(1) == 1 && out.stride(0) >= H * dv &&
               out.scalar_type() == o.scalar_type() && out.device() == o.device(), "kgc.gate_mul: out");
-  kgc::launch_gate_mul(dt_code(o), out.data_ptr(), o.data_ptr(), o.stride(0), o.stride(1),
-                       gt.data_ptr(), gt.stride(0), (int)T, (int)H, (int)dv, stream());
+  kgc::launch_gate_mul(dt_code(o), out.data_ptr(), out.stride(0), o.data_ptr(), o.stride(0),
+                       o.stride(1), gt.data_ptr(), gt.stride(0), (int)T, (int)H, (int)dv,
+                       (float)scale, stream());
 }
 
 void relu_sq(Tensor out, Tensor z) {
@@ -1786,7 +1919,18 @@ TORCH_LIBRARY(kgc, m) {
         "Tensor? seq_lens, Tensor? ctx_lens, Tensor slots, int P, int D, int Tp, int width, bool blocked=True) -> ()");
   m.def("latent_rope_store(Tensor(a!) q_out, Tensor proj, Tensor q_lat, Tensor positions, Tensor? table, "
         "Tensor norm_w, float eps, Tensor(b!) cache, Tensor slots, int H, int d, int r, int rank) -> ()");
-  m.def("gate_mul(Tensor(a!) out, Tensor o, Tensor g) -> ()");
+  m.def("gate_mul(Tensor(a!) out, Tensor o, Tensor g, float scale) -> ()");
+  m.def("causal_conv(Tensor(a!) out, Tensor x, Tensor w, Tensor? bias, Tensor(b!) state, Tensor? qsl, "
+        "Tensor? seq_lens, Tensor? ctx_lens, Tensor slots, Tensor? work_seq, Tensor? work_blk, int P, "
+        "int D, int Tp, bool silu) -> ()");
+  m.def("ssd_scan(Tensor(a!) out, Tensor xbc, Tensor dt, Tensor a_log, Tensor dt_bias, Tensor dskip, "
+        "Tensor(b!) S, Tensor? qsl, Tensor? seq_lens, Tensor? ctx_lens, Tensor slots, int P, int D, "
+        "int Tp, int H, int V, int N, int G) -> ()");
+  m.def("gated_delta_scan(Tensor(a!) out, Tensor qkv, Tensor ba, Tensor a_log, Tensor dt_bias, "
+        "Tensor(b!) S, Tensor? qsl, Tensor? seq_lens, Tensor? ctx_lens, Tensor slots, int P, int D, "
+        "int Tp, int H, int G, int d, int V) -> ()");
+  m.def("gated_rms_norm(Tensor(a!) out, Tensor y, Tensor gate, Tensor w, int groups, float eps, "
+        "bool gate_first) -> ()");
   m.def("relu_sq(Tensor(a!) out, Tensor z) -> ()");
   m.def("side_gate(Tensor(a!) out, Tensor pre, Tensor ids, Tensor table, int col0) -> ()");
   m.def("side_input_rows(Tensor(a!)? out, Tensor(b!) x, Tensor? y, Tensor wg, Tensor wp, Tensor ids, "
@@ -1802,10 +1946,11 @@ TORCH_LIBRARY(kgc, m) {
   m.def("gate_proj(Tensor(a!) out, Tensor h, Tensor w, Tensor? bias, int kind_a, int kind_b, int split, "
         "float cap) -> ()");
   m.def("rope_kv_store(Tensor qkv, Tensor positions, Tensor? table, Tensor(a!) q_out, Tensor(b!) k_cache, "
-        "Tensor(c!) v_cache, Tensor slots, int H, int G, int dk, int dv) -> ()");
+        "Tensor(c!) v_cache, Tensor slots, int H, int G, int dk, int dv, bool interleaved) -> ()");
   m.def("window_attention(Tensor(a!) out, Tensor q, Tensor k_cache, Tensor v_cache, Tensor? qsl, "
         "Tensor? seq_lens, Tensor? pbt, Tensor? ctx_lens, Tensor? dbt, Tensor? work_seq, Tensor? work_blk, "
-        "int P, int D, int Tp, float scale, int window, int keep_first, Tensor? gate, bool fast) -> ()");
+        "int P, int D, int Tp, float scale, int window, int keep_first, Tensor? gate, bool fast, "
+        "float softcap, float out_scale) -> ()");
   m.def("mlstm_scan(Tensor(a!) out, Tensor qkvg, Tensor gates, Tensor(b!) S, Tensor(c!) n, Tensor(d!) m, "
         "Tensor? qsl, Tensor? seq_lens, Tensor? ctx_lens, Tensor slots, int P, int D, int Tp, int H, int d, "
         "int dv) -> ()");
@@ -1930,6 +2075,10 @@ TORCH_LIBRARY_IMPL(kgc, CUDA, m) {
   m.impl("mingru_scan", &mingru_scan);
   m.impl("latent_rope_store", &latent_rope_store);
   m.impl("gate_mul", &gate_mul);
+  m.impl("causal_conv", &causal_conv);
+  m.impl("ssd_scan", &ssd_scan);
+  m.impl("gated_delta_scan", &gated_delta_scan);
+  m.impl("gated_rms_norm", &gated_rms_norm);
   m.impl("relu_sq", &relu_sq);
   m.impl("side_gate", &side_gate);
   m.impl("side_input_rows", &side_input_rows);

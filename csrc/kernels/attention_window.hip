@@ -4,8 +4,9 @@
 // the values may be columns of the key rows (one latent cache row per token).  Query i sees key j when j <= i and (i - j < window or j < keep_first);
 // window <= 0 means plain causal attention.
 //
-//   rope_kv_store     rotates q and k on the first `rot` dims of a head (pair i, i + rot/2;
-//                     cos / sin from an fp32 table), writes q, and k / v into the cache
+//   rope_kv_store     rotates q and k on the first `rot` dims of a head (pair i, i + rot/2,
+//                     or 2i, 2i + 1; cos / sin from an fp32 table), writes q, and k / v
+//                     into the cache
 //   window_attention  one wave per (token, query head): the token's visible keys are the
 //                     kept first tokens plus the window, walked 64 keys at a time (one key
 //                     per lane for the scores, one value column per lane for P.V) with an
@@ -24,7 +25,7 @@ __global__ __launch_bounds__(256) void rope_kv_store_kernel(
     const T* __restrict__ qkv, int64_t qkv_stride, const int64_t* __restrict__ positions,
     const float* __restrict__ table, int rot, int table_rows, T* __restrict__ q_out,
     T* __restrict__ k_cache, T* __restrict__ v_cache, const int64_t* __restrict__ slots, int H,
-    int G, int dk, int dv, int bs, int num_blocks) {
+    int G, int dk, int dv, int bs, int num_blocks, bool interleaved) {
   const int64_t t = blockIdx.x;
   const T* row = qkv + t * qkv_stride;
   int64_t pos = positions[t];
@@ -41,12 +42,15 @@ __global__ __launch_bounds__(256) void rope_kv_store_kernel(
     const int head = e / dk, i = e - head * dk;
     float v = to_f(row[e]);
     if (i < rot) {
-      const int p = i < half ? i : i - half;
+      // pair p: dims (p, p + rot/2), or (2p, 2p + 1) when interleaved
+      const int p = interleaved ? i >> 1 : (i < half ? i : i - half);
+      const bool first = interleaved ? !(i & 1) : i < half;
+      const int ia = interleaved ? 2 * p : p, ib = interleaved ? 2 * p + 1 : half + p;
       const float c = cs[p], sn = cs[half + p];
-      const float a = to_f(row[head * dk + p]), b = to_f(row[head * dk + half + p]);
+      const float a = to_f(row[head * dk + ia]), b = to_f(row[head * dk + ib]);
       float oa, ob;
       neox_rot(a, b, c, sn, oa, ob);
-      v = i < half ? oa : ob;
+      v = first ? oa : ob;
     }
     if (head < H) {
       q_out[(t * H + head) * dk + i] = from_f<T>(v);
@@ -65,6 +69,11 @@ __global__ __launch_bounds__(256) void rope_kv_store_kernel(
 
 constexpr int MAX_DV_PER_LANE = 16;    // dv <= 1024
 
+// scaled score -> cap * tanh(score / cap) when a cap is set
+__device__ __forceinline__ float cap_score(float s, float cap) {
+  return cap > 0.f ? cap * tanhf(s / cap) : s;
+}
+
 // grid (T, H), one wave.  LDS: q row [dk] fp32, p [64], value-row offsets [64].
 template <typename T>
 __global__ __launch_bounds__(64) void window_attention_kernel(
@@ -72,7 +81,8 @@ __global__ __launch_bounds__(64) void window_attention_kernel(
     const T* __restrict__ v_cache, const int* __restrict__ qsl, const int* __restrict__ seq_lens,
     const int* __restrict__ pbt, const int* __restrict__ ctx_lens, const int* __restrict__ dbt,
     int bt_stride, int P, int Tp, int H, int G, int dk, int dv, int krs, int vrs, int bs,
-    int num_blocks, float scale, int window, int keep_first, const float* __restrict__ gate, int kinds) {
+    int num_blocks, float scale, int window, int keep_first, const float* __restrict__ gate, int kinds,
+    WindowExtra ex) {
   extern __shared__ float lds[];
   if (!(kinds & (blockIdx.x < Tp ? 1 : 2))) return;   // rows another kernel of the step owns
   float* qs = lds;                  // [dk]
@@ -80,7 +90,7 @@ __global__ __launch_bounds__(64) void window_attention_kernel(
   int* voff = (int*)(pw + 64);      // [64] (block * G + g) * bs + row
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int g = h / (H / G);
-  T* orow = out + ((int64_t)t * H + h) * dv;
+  T* orow = out + (int64_t)t * ex.ors + h * dv;
   int pos;
   const int* bt;
   if (t < Tp) {
@@ -123,7 +133,7 @@ __global__ __launch_bounds__(64) void window_attention_kernel(
       const T* kr = k_cache + (int64_t)ro * krs;
       float d = 0.f;
       for (int c = 0; c < dk; ++c) d += qs[c] * to_f(kr[c]);
-      s = d * scale;
+      s = cap_score(d * scale, ex.softcap);
     }
     const float mn = fmaxf(m, wave_max(s));
     const float alpha = expf(m - mn);             // m = -inf at first: exp(-inf) = 0
@@ -145,7 +155,7 @@ __global__ __launch_bounds__(64) void window_attention_kernel(
       }
     }
   }
-  const float gt = gate != nullptr ? gate[(int64_t)t * H + h] : 1.f;
+  const float gt = (gate != nullptr ? gate[(int64_t)t * H + h] : 1.f) * ex.out_scale;
   const float inv = gt / l;
 #pragma unroll
   for (int u = 0; u < MAX_DV_PER_LANE; ++u) {
@@ -228,7 +238,7 @@ __global__ __launch_bounds__(64 * NWV) void window_decode_kernel(
     T* __restrict__ out, const T* __restrict__ q, const T* __restrict__ k_cache,
     const T* __restrict__ v_cache, const int* __restrict__ ctx_lens, const int* __restrict__ dbt,
     int bt_stride, int Tp, int H, int G, int dk, int dv, int krs, int vrs, int bs, int num_blocks,
-    float scale, int window, int keep_first, const float* __restrict__ gate) {
+    float scale, int window, int keep_first, const float* __restrict__ gate, WindowExtra ex) {
   extern __shared__ float lds[];
   const int dd = blockIdx.x, g = blockIdx.y, qpg = H / G, hq0 = blockIdx.z * QH;
   const int nh = min(QH, qpg - hq0);
@@ -244,7 +254,7 @@ __global__ __launch_bounds__(64 * NWV) void window_decode_kernel(
   const int* bt = dbt + (int64_t)dd * bt_stride;
   if (pos < 0 || pos >= bt_stride * bs) {             // a padding row: zeros
     for (int e = threadIdx.x; e < nh * dv; e += 64 * NWV)
-      out[((int64_t)t * H + h0) * dv + e] = from_f<T>(0.f);
+      out[(int64_t)t * ex.ors + h0 * dv + e] = from_f<T>(0.f);
     return;
   }
   for (int e = threadIdx.x; e < nh * dk; e += 64 * NWV)
@@ -311,7 +321,7 @@ __global__ __launch_bounds__(64 * NWV) void window_decode_kernel(
     float alpha[QH];
 #pragma unroll
     for (int h = 0; h < QH; ++h) {
-      const float sv = ok ? sc[h] * scale : -INFINITY;
+      const float sv = ok ? cap_score(sc[h] * scale, ex.softcap) : -INFINITY;
       const float mn = fmaxf(m[h], wave_max(sv));
       alpha[h] = expf(m[h] - mn);
       const float p = ok ? expf(sv - mn) : 0.f;
@@ -450,8 +460,8 @@ __global__ __launch_bounds__(64 * NWV) void window_decode_kernel(
       const float mw = mm[w * QH + h];
       if (mw != -INFINITY) L += ml[w * QH + h] * expf(mw - M);
     }
-    const float gt = gate != nullptr ? gate[(int64_t)t * H + h0 + h] : 1.f;
-    out[((int64_t)t * H + h0) * dv + e] = from_f<T>(accs[e] * gt / L);
+    const float gt = (gate != nullptr ? gate[(int64_t)t * H + h0 + h] : 1.f) * ex.out_scale;
+    out[(int64_t)t * ex.ors + h0 * dv + e] = from_f<T>(accs[e] * gt / L);
   }
 }
 
@@ -475,7 +485,8 @@ __global__ __launch_bounds__(256, KSM <= 4 ? 3 : 2) void window_prefill_mfma_ker
     const T* __restrict__ v_cache, const int* __restrict__ qsl, const int* __restrict__ seq_lens,
     const int* __restrict__ pbt, int bt_stride, const int* __restrict__ work_seq,
     const int* __restrict__ work_blk, int blk_rows, int H, int G, int dk, int dv, int krs,
-    int vrs, int bs, int num_blocks, float scale, int window, int keep_first, const float* __restrict__ gate) {
+    int vrs, int bs, int num_blocks, float scale, int window, int keep_first, const float* __restrict__ gate,
+    WindowExtra ex) {
   typedef typename Vec8<T>::type V8;
   extern __shared__ float lds_f[];
   T* Ks = reinterpret_cast<T*>(lds_f);                 // [64][dk + 8]
@@ -586,7 +597,7 @@ __global__ __launch_bounds__(256, KSM <= 4 ? 3 : 2) void window_prefill_mfma_ker
       for (int j = 0; j < 4; ++j)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          s[j][i] *= scale;
+          s[j][i] = cap_score(s[j][i] * scale, ex.softcap);
           tmax = fmaxf(tmax, s[j][i]);
         }
     } else {
@@ -597,7 +608,7 @@ __global__ __launch_bounds__(256, KSM <= 4 ? 3 : 2) void window_prefill_mfma_ker
           const int key = kb + (j >> 1) * 32 + 8 * qd + 4 * (j & 1) + i;
           const bool vis = rowok && key < hi && key <= qpos &&
                            (window <= 0 || qpos - key < window || key < keep_first);
-          s[j][i] = vis ? s[j][i] * scale : -INFINITY;
+          s[j][i] = vis ? cap_score(s[j][i] * scale, ex.softcap) : -INFINITY;
           tmax = fmaxf(tmax, s[j][i]);
         }
     }
@@ -644,9 +655,9 @@ __global__ __launch_bounds__(256, KSM <= 4 ? 3 : 2) void window_prefill_mfma_ker
   l += __shfl_xor(l, 16, 64);
   l += __shfl_xor(l, 32, 64);
   if (rowok) {
-    const float gt = gate != nullptr ? gate[(int64_t)(q0 + myrow) * H + h] : 1.f;
+    const float gt = (gate != nullptr ? gate[(int64_t)(q0 + myrow) * H + h] : 1.f) * ex.out_scale;
     const float inv = l > 0.f ? gt / l : 0.f;
-    T* orow = out + ((int64_t)(q0 + myrow) * H + h) * dv;
+    T* orow = out + (int64_t)(q0 + myrow) * ex.ors + h * dv;
 #pragma unroll
     for (int t2 = 0; t2 < DTM; ++t2) {
       if (t2 < ndt) {
@@ -671,11 +682,12 @@ __global__ __launch_bounds__(256, KSM <= 4 ? 3 : 2) void window_prefill_mfma_ker
 void launch_rope_kv_store(int dtype, const void* qkv, int64_t qkv_stride,
                           const int64_t* positions, const float* table, int rot, int table_rows,
                           void* q_out, void* k_cache, void* v_cache, const int64_t* slots, int T_,
-                          int H, int G, int dk, int dv, int bs, int num_blocks, hipStream_t s) {
+                          int H, int G, int dk, int dv, int bs, int num_blocks, bool interleaved,
+                          hipStream_t s) {
   if (T_ <= 0) return;
   KGC_DISPATCH_T(dtype, rope_kv_store_kernel<T><<<T_, 256, 0, s>>>(
       (const T*)qkv, qkv_stride, positions, table, rot, table_rows, (T*)q_out, (T*)k_cache,
-      (T*)v_cache, slots, H, G, dk, dv, bs, num_blocks));
+      (T*)v_cache, slots, H, G, dk, dv, bs, num_blocks, interleaved));
 }
 
 int window_attention_max_dv() { return 64 * MAX_DV_PER_LANE; }
@@ -685,13 +697,13 @@ void launch_window_attention(int dtype, void* out, const void* q, const void* k_
                              const int* pbt, const int* ctx_lens, const int* dbt, int bt_stride,
                              int P, int Tp, int T_, int H, int G, int dk, int dv, int krs, int vrs,
                              int bs, int num_blocks, float scale, int window, int keep_first,
-                             const float* gate, int kinds, hipStream_t s) {
+                             const float* gate, int kinds, WindowExtra ex, hipStream_t s) {
   if (T_ <= 0 || !kinds) return;
   const size_t lds = (size_t)(dk + 128) * sizeof(float);
   KGC_DISPATCH_T(dtype, window_attention_kernel<T><<<dim3(T_, H), 64, lds, s>>>(
       (T*)out, (const T*)q, (const T*)k_cache, (const T*)v_cache, qsl, seq_lens, pbt, ctx_lens,
       dbt, bt_stride, P, Tp, H, G, dk, dv, krs, vrs, bs, num_blocks, scale, window, keep_first,
-      gate, kinds));
+      gate, kinds, ex));
 }
 
 // decode rows on the 8-wave kernel: needs 16-byte key rows (dk % 8 == 0), even dv <= 512
@@ -709,7 +721,7 @@ template <typename T>
 static void decode_dispatch(T* out, const T* q, const T* kc, const T* vc, const int* ctx_lens,
                             const int* dbt, int bt_stride, int Tp, int D, int H, int G, int dk,
                             int dv, int krs, int vrs, int bs, int num_blocks, float scale, int window,
-                            int keep_first, const float* gate, hipStream_t s) {
+                            int keep_first, const float* gate, WindowExtra ex, hipStream_t s) {
   const int qpg = H / G;
   int QH = qpg >= 8 ? 8 : qpg >= 3 ? 4 : qpg;            // heads per workgroup: 1, 2, 4, 8
   // many heads on one key/value group and few rows: smaller head groups, so that the grid
@@ -722,7 +734,7 @@ static void decode_dispatch(T* out, const T* q, const T* kc, const T* vc, const 
 #define KGC_DEC(N, W)                                                                        \
   window_decode_kernel<T, N, W><<<grid, 64 * W, decode_lds(N, W, dk, dv), s>>>(              \
       out, q, kc, vc, ctx_lens, dbt, bt_stride, Tp, H, G, dk, dv, krs, vrs, bs, num_blocks,     \
-      scale, window, keep_first, gate)
+      scale, window, keep_first, gate, ex)
 #define KGC_DEC2(N) \
   do {              \
     if (small) KGC_DEC(N, 4); else KGC_DEC(N, 8); \
@@ -744,12 +756,12 @@ void launch_window_decode(int dtype, void* out, const void* q, const void* k_cac
                           const void* v_cache, const int* ctx_lens, const int* dbt,
                           int bt_stride, int Tp, int D, int H, int G, int dk, int dv, int krs,
                           int vrs, int bs, int num_blocks, float scale, int window, int keep_first,
-                          const float* gate, hipStream_t s) {
+                          const float* gate, WindowExtra ex, hipStream_t s) {
   if (D <= 0) return;
   KGC_DISPATCH_T(dtype, decode_dispatch<T>((T*)out, (const T*)q, (const T*)k_cache,
                                            (const T*)v_cache, ctx_lens, dbt, bt_stride, Tp, D, H,
                                            G, dk, dv, krs, vrs, bs, num_blocks, scale, window, keep_first,
-                                           gate, s));
+                                           gate, ex, s));
 }
 
 size_t window_prefill_mfma_lds(int dk, int dv) {
@@ -769,13 +781,13 @@ static void prefill_dispatch(T* out, const T* q, const T* kc, const T* vc, const
                              const int* work_seq, const int* work_blk, int n_work, int blk_rows,
                              int H, int G, int dk, int dv, int krs, int vrs, int bs, int num_blocks,
                              float scale, int window, int keep_first, const float* gate,
-                             hipStream_t s) {
+                             WindowExtra ex, hipStream_t s) {
   const dim3 grid(n_work * (blk_rows / PFW_BM), H);
   const size_t lds = window_prefill_mfma_lds(dk, dv);
 #define KGC_PF(K, D)                                                                          \
   window_prefill_mfma_kernel<T, K, D><<<grid, 256, lds, s>>>(                                 \
       out, q, kc, vc, qsl, seq_lens, pbt, bt_stride, work_seq, work_blk, blk_rows, H, G, dk,  \
-      dv, krs, vrs, bs, num_blocks, scale, window, keep_first, gate)
+      dv, krs, vrs, bs, num_blocks, scale, window, keep_first, gate, ex)
   if (dk <= 128 && dv <= 128) KGC_PF(4, 8);
   else KGC_PF(8, 16);
 #undef KGC_PF
@@ -786,17 +798,17 @@ void launch_window_prefill_mfma(int dtype, void* out, const void* q, const void*
                                 const int* pbt, int bt_stride, const int* work_seq,
                                 const int* work_blk, int n_work, int blk_rows, int H, int G,
                                 int dk, int dv, int krs, int vrs, int bs, int num_blocks, float scale, int window,
-                                int keep_first, const float* gate, hipStream_t s) {
+                                int keep_first, const float* gate, WindowExtra ex, hipStream_t s) {
   if (n_work <= 0) return;
   if (dtype == DT_BF16)
     prefill_dispatch<bf16>((bf16*)out, (const bf16*)q, (const bf16*)k_cache,
                            (const bf16*)v_cache, qsl, seq_lens, pbt, bt_stride, work_seq,
                            work_blk, n_work, blk_rows, H, G, dk, dv, krs, vrs, bs, num_blocks,
-                           scale, window, keep_first, gate, s);
+                           scale, window, keep_first, gate, ex, s);
   else
     prefill_dispatch<f16>((f16*)out, (const f16*)q, (const f16*)k_cache, (const f16*)v_cache,
                           qsl, seq_lens, pbt, bt_stride, work_seq, work_blk, n_work, blk_rows, H,
-                          G, dk, dv, krs, vrs, bs, num_blocks, scale, window, keep_first, gate, s);
+                          G, dk, dv, krs, vrs, bs, num_blocks, scale, window, keep_first, gate, ex, s);
 }
 
 // ---- latent attention: cache rows [normed latent | rotary key part] and query rows --------

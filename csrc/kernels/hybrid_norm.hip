@@ -115,6 +115,7 @@ __global__ __launch_bounds__(NT) void xielu_kernel(T* __restrict__ out, const T*
 
 __device__ __forceinline__ float gate_act(float y, int kind, float cap) {
   if (kind == 0) return 1.f / (1.f + expf(-y));
+  if (kind == 3) return y;                            // the plain projection (router logits)
   y = cap * tanhf(y / cap);
   if (kind == 1) return y;
   // logsigmoid(y) = min(y, 0) - log1p(exp(-|y|))
@@ -361,17 +362,18 @@ __global__ __launch_bounds__(NT) void residual_norm_kernel(
   for (int c = threadIdx.x; c < W; c += NT) o[c] = from_f<O>(xr[c] * r * w[c]);
 }
 
-// out [T, H * dv] = o[t, h, :] (strides st, sh) * sigmoid(g[t, h * dv + :]) (row stride sg)
+// out [T, H * dv] (row stride so) = o[t, h, :] (strides st, sh) * sigmoid(g[t, h * dv + :])
+// (row stride sg) * scale
 template <typename T>
 __global__ __launch_bounds__(NT) void gate_mul_kernel(
-    T* __restrict__ out, const T* __restrict__ o, int64_t st, int64_t sh,
-    const T* __restrict__ g, int64_t sg, int H, int dv) {
+    T* __restrict__ out, int64_t so, const T* __restrict__ o, int64_t st, int64_t sh,
+    const T* __restrict__ g, int64_t sg, int H, int dv, float scale) {
   const int64_t t = blockIdx.x;
   const int n = H * dv;
   for (int e = threadIdx.x; e < n; e += NT) {
     const int h = e / dv, c = e - h * dv;
     const float gate = 1.f / (1.f + expf(-to_f(g[t * sg + e])));
-    out[t * n + e] = from_f<T>(to_f(o[t * st + h * sh + c]) * gate);
+    out[t * so + e] = from_f<T>(to_f(o[t * st + h * sh + c]) * gate * scale);
   }
 }
 
@@ -565,11 +567,12 @@ void launch_residual_norm(int dtype, int out_dtype, void* out, float* x, const v
 #undef KGC_RN
 }
 
-void launch_gate_mul(int dtype, void* out, const void* o, int64_t st, int64_t sh, const void* g,
-                     int64_t sg, int rows, int H, int dv, hipStream_t s) {
+void launch_gate_mul(int dtype, void* out, int64_t so, const void* o, int64_t st, int64_t sh,
+                     const void* g, int64_t sg, int rows, int H, int dv, float scale,
+                     hipStream_t s) {
   if (rows <= 0) return;
-  KGC_DISPATCH_T(dtype, gate_mul_kernel<T><<<rows, NT, 0, s>>>((T*)out, (const T*)o, st, sh,
-                                                              (const T*)g, sg, H, dv));
+  KGC_DISPATCH_T(dtype, gate_mul_kernel<T><<<rows, NT, 0, s>>>((T*)out, so, (const T*)o, st, sh,
+                                                              (const T*)g, sg, H, dv, scale));
 }
 
 void launch_relu_sq(int dtype, void* out, const void* z, int64_t n, hipStream_t s) {

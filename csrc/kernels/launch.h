@@ -266,14 +266,23 @@ void launch_gate_proj(int dtype, float* out, const void* h, const void* w, const
 void launch_rope_kv_store(int dtype, const void* qkv, int64_t qkv_stride,
                           const int64_t* positions, const float* table, int rot, int table_rows,
                           void* q_out, void* k_cache, void* v_cache, const int64_t* slots, int T,
-                          int H, int G, int dk, int dv, int bs, int num_blocks, hipStream_t s);
+                          int H, int G, int dk, int dv, int bs, int num_blocks, bool interleaved,
+                          hipStream_t s);
 int window_attention_max_dv();
+// what an attention inside a wider mixer adds: the row stride of `out` in elements (its
+// rows may be column slices of a wider buffer), a tanh cap on the scaled scores (<= 0:
+// none), a factor on the result
+struct WindowExtra {
+  int64_t ors;
+  float softcap;
+  float out_scale;
+};
 void launch_window_attention(int dtype, void* out, const void* q, const void* k_cache,
                              const void* v_cache, const int* qsl, const int* seq_lens,
                              const int* pbt, const int* ctx_lens, const int* dbt, int bt_stride,
                              int P, int Tp, int T, int H, int G, int dk, int dv, int krs, int vrs,
                              int bs, int num_blocks, float scale, int window, int keep_first,
-                             const float* gate, int kinds, hipStream_t s);
+                             const float* gate, int kinds, WindowExtra ex, hipStream_t s);
 // `kinds` above: bit 0 = run the prefill rows, bit 1 = run the decode rows (the simple kernel
 // covers whatever the two kernels below do not take)
 bool window_decode_ok(int dk, int dv, int qpg);
@@ -282,14 +291,14 @@ void launch_window_decode(int dtype, void* out, const void* q, const void* k_cac
                           const void* v_cache, const int* ctx_lens, const int* dbt,
                           int bt_stride, int Tp, int D, int H, int G, int dk, int dv, int krs,
                           int vrs, int bs, int num_blocks, float scale, int window, int keep_first,
-                          const float* gate, hipStream_t s);
+                          const float* gate, WindowExtra ex, hipStream_t s);
 bool window_prefill_mfma_ok(int dtype, int dk, int dv);
 void launch_window_prefill_mfma(int dtype, void* out, const void* q, const void* k_cache,
                                 const void* v_cache, const int* qsl, const int* seq_lens,
                                 const int* pbt, int bt_stride, const int* work_seq,
                                 const int* work_blk, int n_work, int blk_rows, int H, int G,
                                 int dk, int dv, int krs, int vrs, int bs, int num_blocks, float scale, int window,
-                                int keep_first, const float* gate, hipStream_t s);
+                                int keep_first, const float* gate, WindowExtra ex, hipStream_t s);
 int mlstm_scan_max_dim();
 void launch_mlstm_scan(int dtype, float* out, const void* qkvg, int64_t stride,
                        const float* gates, float* S, float* nst, float* mst, const int* qsl,
@@ -301,8 +310,9 @@ void launch_mlstm_scan(int dtype, float* out, const void* qkvg, int64_t stride,
 void launch_residual_norm(int dtype, int out_dtype, void* out, float* x, const void* add,
                           const float* anw, const float* w, float mult, int rows, int W,
                           float eps, hipStream_t s);
-void launch_gate_mul(int dtype, void* out, const void* o, int64_t st, int64_t sh, const void* g,
-                     int64_t sg, int rows, int H, int dv, hipStream_t s);
+void launch_gate_mul(int dtype, void* out, int64_t so, const void* o, int64_t st, int64_t sh,
+                     const void* g, int64_t sg, int rows, int H, int dv, float scale,
+                     hipStream_t s);
 void launch_relu_sq(int dtype, void* out, const void* z, int64_t n, hipStream_t s);
 void launch_side_gate(int dtype, void* out, const void* pre, const int64_t* ids,
                       const void* table, int64_t ts, int vocab, int col0, int rows, int n,
@@ -336,5 +346,29 @@ void launch_moe_route_sigmoid(float* w, int* ids, const float* scores, int64_t s
 void launch_moe_finish(int dtype, void* out, const void* routed, const void* dense,
                        const float* w, const int* ids, const void* shared, const float* gate,
                        int64_t gs, int ntok, int E, int k, int W, hipStream_t s);
+
+// ---- parallel mixers (parallel_mixer.hip): convolution state, Mamba-2, gated delta rule ----
+// `dtype`: activation type of the projection columns read (x / dt / ba / gate) and of the
+// gated norm's output; convolution and scan outputs are fp32
+int causal_conv_max_taps();
+void launch_causal_conv(int dtype, float* out, const void* x, int64_t xs, const float* w,
+                        const float* bias, float* state, const int* qsl, const int* seq_lens,
+                        const int* ctx_lens, const int* slots, const int* work_seq,
+                        const int* work_blk, int n_work, int blk_rows, int P, int D, int Tp,
+                        int C, int K, int num_slots, bool silu, hipStream_t s);
+int matrix_scan_max_rows();
+void launch_ssd_scan(int dtype, float* out, const float* xbc, const void* dt, int64_t dts,
+                     const float* a_log, const float* dt_bias, const float* dskip, float* S,
+                     const int* qsl, const int* seq_lens, const int* ctx_lens, const int* slots,
+                     int P, int D, int Tp, int H, int V, int N, int G, int num_slots,
+                     hipStream_t s);
+void launch_gated_delta_scan(int dtype, float* out, const float* qkv, const void* ba,
+                             int64_t bas, const float* a_log, const float* dt_bias, float* S,
+                             const int* qsl, const int* seq_lens, const int* ctx_lens,
+                             const int* slots, int P, int D, int Tp, int H, int G, int d, int V,
+                             int num_slots, hipStream_t s);
+void launch_gated_rms_norm(int dtype, void* out, int64_t os, const float* y, const void* gate,
+                           int64_t gs, const float* w, int rows, int n, int groups, float eps,
+                           bool gate_first, hipStream_t s);
 
 }  // namespace kgc

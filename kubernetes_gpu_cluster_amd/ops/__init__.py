@@ -988,8 +988,15 @@ def causal_conv(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor],
     if not _gpu(x):
         return ref.causal_conv(x, w, bias, state, ref.step_sequences(meta), silu)
     out = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+    ws, wb = getattr(meta, "work_seq", None), getattr(meta, "work_mblk", None)
+    if meta.num_prefills and ws is None:
+        qsl = meta.query_start_loc.tolist()
+        a, b = prefill_work_list([qsl[i + 1] - qsl[i] for i in range(meta.num_prefills)],
+                                 meta.prefill_seq_lens.tolist())
+        ws = torch.tensor(a, dtype=torch.int32, device=x.device)
+        wb = torch.tensor(b, dtype=torch.int32, device=x.device)
     _k().causal_conv(out, x, w, bias, state, meta.query_start_loc, meta.prefill_seq_lens,
-                     meta.decode_ctx_lens, meta.state_slots, meta.num_prefills,
+                     meta.decode_ctx_lens, meta.state_slots, ws, wb, meta.num_prefills,
                      meta.num_decodes, meta.num_prefill_tokens, silu)
     return out
 

@@ -735,7 +735,7 @@ def causal_conv(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor],
     for a, n, p0, slot in seqs:
         if slot < 0:
             continue
-        prev = torch.zeros(K - 1, C) if p0 == 0 else state[slot].clone()
+        prev = torch.zeros(K - 1, C) if p0 == 0 else state[slot][: K - 1].clone()
         xs = torch.cat([prev, x[a:a + n].float()], 0)              # [K-1+n, C]
         y = torch.zeros(n, C)
         for j in range(K):
