@@ -403,6 +403,60 @@ PRESETS.update({
 })
 
 
+def _nolesun(name: str, width: int, pattern: str, att: dict, ssm: dict, gdn: dict, dense_ff: int,
+             expert_ff: int, loop: Optional[tuple], experts: int = 8, top: int = 2,
+             vocab: int = 32000) -> ModelConfig:
+    """A Nolesun-architecture preset: ``pattern`` is one letter per layer ("m": attention
+    beside Mamba-2, "d": biased, capped, gated attention beside the gated delta rule; a
+    capital letter: routed experts instead of the dense feed-forward)."""
+    dense = FeedForwardSpec("dense", dense_ff, act="relu2", gated=False)
+    moe = FeedForwardSpec("moe", expert_ff, act="silu", gated=True, experts=experts, top=top,
+                          router="softmax")
+    specs = []
+    for c in pattern:
+        two = c.lower() == "d"
+        rs = RotarySpec(att["rot"], att.get("base", 1e4), interleaved=two)
+        left = MixerSpec("attention", att["heads"], att["dim"], att["vdim"], kv_heads=att["kv"],
+                         scale=att["dim"] ** -0.5, rot_dims=rs.dims, rot_base=rs.base, rotary=rs,
+                         bias=two, softcap=30.0 if two else 0.0, elem_gate=two)
+        right = (MixerSpec("gated_delta", gdn["heads"], gdn["dim"], gdn["vdim"], kv_heads=gdn["kv"],
+                           conv=gdn.get("conv", 4)) if two else
+                 MixerSpec("mamba2", ssm["heads"], ssm["state"], ssm["vdim"],
+                           kv_heads=ssm.get("groups", 1), conv=ssm.get("conv", 4),
+                           inner_norm_groups=ssm.get("norm_groups", 1)))
+        mlp = moe if c.isupper() else dense
+        specs.append(MixerSpec("parallel", left.heads, left.dim, left.vdim, kv_heads=left.kv_heads,
+                               ff=mlp.ff, mlp=mlp, left=left, right=right,
+                               left_scale=1.0, right_scale=1.0))
+    return ModelConfig(name, "nolesun", len(specs), width, att["heads"], att["kv"], att["dim"],
+                       dense_ff, vocab, max_position=8192, rms_eps=1e-6, layer_specs=tuple(specs),
+                       embed_scale=width ** 0.5, layer_loop=loop, loop_mix=loop is not None,
+                       bos_token_id=1, eos_token_id=2)
+
+
+# Nolesun presets beside the equal-width hybrid / Llama presets above: the same number of
+# layer runs (a looped pair counts twice), 16 / 32 attention heads of 128, and a feed-forward
+# whose active parameters per token are those of the Llama preset's (the two-matrix dense one
+# 1.5 x as wide as the gated one; two of eight gated experts of half its size).  Every layer
+# also carries a recurrence as wide as the model (Mamba-2: heads of 64 with a state of 128;
+# gated delta rule: heads of 128 x 128), so a layer has about twice a Llama layer's mixer.
+PRESETS.update({
+    "nolesun-w2048": _nolesun("nolesun-w2048", 2048, "mDmDmDmDmD",
+                              dict(heads=16, kv=4, dim=128, vdim=128, rot=64),
+                              dict(heads=32, vdim=64, state=128, groups=1),
+                              dict(heads=16, kv=8, dim=128, vdim=128), 8256, 2752, (2, 4, 2)),
+    "nolesun-w4096": _nolesun("nolesun-w4096", 4096, "mDmDmD",
+                              dict(heads=32, kv=8, dim=128, vdim=128, rot=64),
+                              dict(heads=64, vdim=64, state=128, groups=1),
+                              dict(heads=32, kv=16, dim=128, vdim=128), 21504, 7168, (2, 4, 2)),
+    "tiny-nolesun": _nolesun("tiny-nolesun", 128, "mDdM",
+                             dict(heads=4, kv=2, dim=32, vdim=16, rot=16),
+                             dict(heads=4, vdim=16, state=16, groups=2, conv=3, norm_groups=2),
+                             dict(heads=4, kv=2, dim=16, vdim=16, conv=4), 192, 64, (1, 3, 2),
+                             experts=4, vocab=1024),
+})
+
+
 # HF repo basenames (lower-cased) -> preset
 _ALIASES = {
     "meta-llama-3-8b": "llama-3-8b", "meta-llama-3-8b-instruct": "llama-3-8b",

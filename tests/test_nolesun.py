@@ -1,0 +1,539 @@
+"""Nolesun through the engine (registry, safetensors loading, block manager, state slots,
+step packing, kernels) against the plain numpy oracle in ``nolesun_oracle.py``.
+
+Every test writes its own small config.json + model.safetensors (random bf16 weights)
+and drives the engine with the teacher-forced replayer or the generation entry points.
+CPU runs use the reference ops in fp32; ``-m gpu`` runs use the HIP kernels in fp32 and
+bf16.  Pages are 8 tokens, so prompts cross many page borders, and the recurrences carry
+every earlier token: a key wrongly hidden, a lost state, a convolution input taken from the
+wrong step or a skipped pass changes the logits far beyond the tolerances."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import nolesun_oracle as oracle
+from kubernetes_gpu_cluster_amd.engine.config import EngineConfig
+from kubernetes_gpu_cluster_amd.engine.llm_engine import LLM, LLMEngine
+from kubernetes_gpu_cluster_amd.engine.replay import TraceReplayer
+from kubernetes_gpu_cluster_amd.engine.sequence import SamplingParams
+
+CPU = pytest.param("cpu", "float32", id="cpu-fp32")
+GPU32 = pytest.param("cuda", "float32", marks=pytest.mark.gpu, id="gpu-fp32")
+GPU16 = pytest.param("cuda", "bfloat16", marks=pytest.mark.gpu, id="gpu-bf16")
+DEVICES = [CPU, GPU32, GPU16]
+# Row error: rms of the logit difference over the rms of the logits, means taken off.
+# fp32: every row within 3e-4.  bf16: rounding moves a row by a few percent (median within
+# 0.04, every row within 0.3) -- except where rounding flips a routing choice: a token whose
+# router logits the oracle itself separates by less than MARGIN is a close call, and such a
+# row (and, through the recurrent state, the few after it) is only held to 2.0.
+TOL = {"float32": 3e-4, "bfloat16": 0.3}
+TOL_MEDIAN = {"float32": 3e-4, "bfloat16": 0.04}
+MARGIN, AFTER = 0.05, 4
+
+
+def att(heads=4, kv=2, dim=12, vdim=10, rot=8, base=100.0, scale=0.3, softcap=None):
+    m = {"heads": heads, "kv_heads": kv, "dim": dim, "vdim": vdim, "scale": scale,
+         "rot": {"dims": rot, "base": base}}
+    if softcap:
+        m["softcap"] = softcap
+    return m
+
+
+def ssm(heads=4, vdim=8, state=12, groups=2, conv=3, norm_groups=2):
+    return {"heads": heads, "vdim": vdim, "state": state, "groups": groups, "conv": conv,
+            "norm_groups": norm_groups}
+
+
+def delta(heads=4, kv=2, dim=10, vdim=6, conv=4):
+    return {"heads": heads, "kv_heads": kv, "dim": dim, "vdim": vdim, "conv": conv}
+
+
+def par(left, right, mlp=None, ls=1.2, rs=0.9):
+    return {"type": "parallel", "mixer": {"left": left, "right": right, "left_scale": ls,
+                                          "right_scale": rs}, "mlp": mlp}
+
+
+def par2(left, right, mlp=None, ls=0.7, rs=1.3):
+    return {"type": "parallel_2", "mixer": {"left": left, "right": right, "left_scale": ls,
+                                            "right_scale": rs}, "mlp": mlp}
+
+
+def dense(ff=48):
+    return {"kind": "dense", "ff": ff}
+
+
+def moe(experts=6, top=2, ff=20):
+    return {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "top": top}}
+
+
+def config(layers, width=64, vocab=160, eps=1e-5, loop=None, scale=3.0):
+    c = {"architecture": "Nolesun", "vocab": vocab, "width": width, "layers": layers,
+         "norm": {"eps": eps}, "embedding": {"scale": scale}}
+    if loop:
+        c["loop"] = dict(zip(("start", "stop", "times"), loop))
+    return c
+
+
+MIXED = config([par(att(), ssm(), dense()), par2(att(softcap=4.0), delta(), moe()),
+                par(att(heads=3, kv=1, dim=8, vdim=16, rot=4, scale=0.4),
+                    ssm(heads=2, vdim=12, state=6, groups=1, conv=2, norm_groups=1), moe(top=3)),
+                par2(att(heads=2, kv=2, dim=16, vdim=8, rot=16, softcap=9.0),
+                     delta(heads=2, kv=1, dim=8, vdim=8, conv=3))], loop=(1, 3, 2))
+# values a model may make equal or 1, and parts it may leave out: one head, one group, one
+# expert used of two, no loop, no feed-forward, rotary over the whole head or over two
+# dimensions, scales of 1, a convolution of two taps, value size = key size = state size
+PLAIN = config([par2(att(heads=1, kv=1, dim=16, vdim=16, rot=16, scale=0.25, softcap=30.0),
+                     delta(heads=1, kv=1, dim=16, vdim=16, conv=2), dense(32), ls=1.0, rs=1.0),
+                par(att(heads=2, kv=2, dim=8, vdim=8, rot=2), ssm(heads=1, vdim=16, state=16,
+                                                                  groups=1, conv=2, norm_groups=1),
+                    moe(experts=2, top=1, ff=16), ls=1.0, rs=1.0),
+                par(att(heads=2, kv=1, dim=8, vdim=8, rot=8),
+                    ssm(heads=2, vdim=8, state=8, groups=2, conv=4, norm_groups=2))],
+               width=48, vocab=96, scale=1.0)
+# sizes the matrix-core prefill kernel, the 16-byte decode paths and the grouped expert GEMM
+# take (heads of 64 and 32 with values of 32 and 64; experts of 64 on a width of 128; states
+# of 64 x 64 and 32 x 64), prompts over several key tiles and row blocks, the whole stack
+# looped three times
+WIDE = config([par(att(heads=8, kv=2, dim=64, vdim=32, rot=32, scale=0.12),
+                   ssm(heads=4, vdim=64, state=64, groups=2, conv=4, norm_groups=2),
+                   moe(experts=8, top=3, ff=64)),
+               par2(att(heads=4, kv=4, dim=32, vdim=64, rot=32, scale=0.15, softcap=15.0, base=500.0),
+                    delta(heads=4, kv=2, dim=32, vdim=64, conv=4), dense(96))],
+              width=128, vocab=200, loop=(0, 2, 3), scale=8.0)
+# sizes that are multiples of nothing: odd vocabulary and width, heads whose bytes are no
+# multiple of 16, five experts, three groups, one layer looped three times at the end
+ODD = config([par(att(heads=3, kv=3, dim=10, vdim=14, rot=6, base=30.0, scale=0.35),
+                  ssm(heads=6, vdim=5, state=9, groups=3, conv=5, norm_groups=3), moe(experts=5, top=2, ff=18)),
+              par2(att(heads=6, kv=2, dim=6, vdim=4, rot=2, scale=0.5, softcap=2.5),
+                   delta(heads=6, kv=3, dim=7, vdim=11, conv=3), dense(26))],
+             width=70, vocab=251, eps=1e-6, loop=(1, 2, 3), scale=0.5)
+
+
+def write_model(path, cfg, seed):
+    """Random bf16 weights in the checkpoint's naming; returns them as float64 arrays."""
+    from safetensors.torch import save_file
+    g = torch.Generator().manual_seed(seed)
+    W = cfg["width"]
+    t = {}
+
+    def lin(name, out, inp, gain=1.0):
+        t[name] = torch.randn(out, inp, generator=g) * gain / inp ** 0.5
+
+    def vec(name, n, base, spread):
+        t[name] = base + spread * torch.randn(n, generator=g)
+    t["embed"] = torch.randn(cfg["vocab"], W, generator=g) * 0.5
+    lin("head", cfg["vocab"], W, 2.0)
+    vec("final.norm", W, 0.0, 0.2)
+    lp = cfg.get("loop")
+    if lp:
+        lin("loop.in", W, 2 * W, 1.5)
+        t["loop.step"] = 0.3 * torch.randn(lp["times"], W, generator=g)
+    for i, lc in enumerate(cfg["layers"]):
+        L, m = "l%d." % i, lc["mixer"]
+        two = lc["type"] == "parallel_2"
+        for n in ("norm1", "norm1b") + (("norm2", "norm2b") if lc["mlp"] else ()):
+            vec(L + n, W, 0.0, 0.2)
+        vec(L + "ls1", W, 0.6, 0.2)
+        a, P = m["left"], L + "mix.left."
+        H, G, d, dv = a["heads"], a["kv_heads"], a["dim"], a["vdim"]
+        lin(P + "q", H * d, W, 2.0)
+        lin(P + "k", G * d, W, 2.0)
+        lin(P + "v", G * dv, W)
+        lin(P + "o", W, H * dv)
+        if two:
+            lin(P + "g", H * dv, W, 2.0)
+            for n, sz in (("q.b", H * d), ("k.b", G * d), ("v.b", G * dv), ("o.b", W)):
+                vec(P + n, sz, 0.0, 0.3)
+        r, P = m["right"], L + "mix.right."
+        if two:
+            H, G, d, dv, K = r["heads"], r["kv_heads"], r["dim"], r["vdim"], r["conv"]
+            for n, sz in (("q", G * d), ("k", G * d), ("v", H * dv)):
+                lin(P + n, sz, W, 2.0)
+                t[P + n + ".conv"] = torch.randn(sz, K, generator=g) * 0.6
+            lin(P + "g", H * dv, W, 2.0)
+            lin(P + "b", H, W, 2.0)
+            lin(P + "a", H, W, 2.0)
+            vec(P + "A_log", H, -0.5, 0.7)
+            vec(P + "dt_bias", H, -1.0, 0.7)
+            vec(P + "norm", dv, 1.0, 0.2)
+            lin(P + "o", W, H * dv)
+        else:
+            H, V, N, G, K = r["heads"], r["vdim"], r["state"], r["groups"], r["conv"]
+            lin(P + "in", 2 * H * V + 2 * G * N + H, W, 2.0)
+            t[P + "conv"] = torch.randn(H * V + 2 * G * N, K, generator=g) * 0.6
+            vec(P + "conv.b", H * V + 2 * G * N, 0.0, 0.3)
+            vec(P + "A_log", H, -0.5, 0.7)
+            vec(P + "dt_bias", H, -1.0, 0.7)
+            vec(P + "D", H, 0.5, 0.5)
+            vec(P + "norm", H * V, 1.0, 0.2)
+            lin(P + "o", W, H * V)
+        f = lc["mlp"]
+        if f:
+            vec(L + "ls2", W, 0.6, 0.2)
+            if f["kind"] == "dense":
+                lin(L + "mlp.up", f["ff"], W, 2.0)
+                lin(L + "mlp.down", W, f["ff"])
+            else:
+                for e in range(f["router"]["experts"]):
+                    lin(L + "mlp.e%d.gate" % e, f["expert"]["ff"], W, 2.0)
+                    lin(L + "mlp.e%d.up" % e, f["expert"]["ff"], W, 2.0)
+                    lin(L + "mlp.e%d.down" % e, W, f["expert"]["ff"])
+                lin(L + "mlp.router", f["router"]["experts"], W, 3.0)
+                vec(L + "mlp.router.b", f["router"]["experts"], 0.0, 0.5)
+    t = {k: v.to(torch.bfloat16).contiguous() for k, v in t.items()}
+    os.makedirs(path, exist_ok=True)
+    save_file(t, os.path.join(path, "model.safetensors"))
+    with open(os.path.join(path, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    return {k: v.double().numpy() for k, v in t.items()}
+
+
+@pytest.fixture(scope="module")
+def models(tmp_path_factory):
+    root = tmp_path_factory.mktemp("nolesun")
+    out = {}
+    for name, cfg, seed in (("mixed", MIXED, 31), ("plain", PLAIN, 32), ("wide", WIDE, 33),
+                            ("odd", ODD, 34)):
+        d = str(root / name)
+        out[name] = (d, cfg, write_model(d, cfg, seed))
+    return out
+
+
+_engines = {}
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _release_engines():
+    """Engines are shared by the tests of this module and released after the last one."""
+    yield
+    for eng in _engines.values():
+        eng.shutdown()
+    _engines.clear()
+    import gc
+    gc.collect()
+    if torch.cuda.is_available():
+        torch.cuda.empty_cache()
+
+
+def engine(models, name, device, dtype, pages=24, page=8, seqs=4, **kw):
+    if device == "cuda" and not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    key = (name, device, dtype, pages, page, seqs, tuple(sorted(kw.items())))
+    if key not in _engines:
+        d = models[name][0]
+        _engines[key] = LLMEngine(EngineConfig(
+            model=d, dtype=dtype, device=device, block_size=page, max_num_seqs=seqs,
+            max_model_len=pages * page, max_num_batched_tokens=pages * page,
+            num_gpu_blocks_override=pages + 1, cuda_graph_max_bs=seqs, **kw))
+    return _engines[key]
+
+
+def row_errs(got, want):
+    got, want = np.asarray(got, dtype=np.float64), np.asarray(want, dtype=np.float64)
+    d = got - want
+    d = d - d.mean(-1, keepdims=True)
+    w = want - want.mean(-1, keepdims=True)
+    return np.sqrt((d ** 2).mean(-1) / (w ** 2).mean(-1))
+
+
+class Verdict:
+    def __init__(self, ok, text):
+        self.ok, self.text = ok, text
+
+    def __bool__(self):
+        return self.ok
+
+    def __repr__(self):
+        return self.text
+
+
+class Expected:
+    def __init__(self, logits, shaky):
+        self.logits, self.shaky = logits, shaky
+
+    def __getitem__(self, key):
+        return Expected(self.logits[key], self.shaky[key])
+
+
+_expected = {}
+
+
+def expected(cfg, wts, toks):
+    """The oracle's logits, with the rows marked whose routing was a close call."""
+    key = (id(wts), tuple(toks))
+    if key not in _expected:
+        margins = []
+        lg = oracle.forward(cfg, wts, toks, margins=margins)
+        shaky = np.zeros(len(toks), dtype=bool)
+        if margins:
+            for t in np.where(np.min(np.stack(margins), axis=0) < MARGIN)[0]:
+                shaky[t:t + 1 + AFTER] = True
+        _expected[key] = Expected(lg, shaky)
+    return _expected[key]
+
+
+def close(got, want, dtype):
+    e = row_errs(got, want.logits)
+    firm = ~want.shaky if dtype != "float32" else np.ones(len(e), dtype=bool)
+    text = "rows %d (%d firm): median %.2g, worst firm %.2g, worst %.2g" % (
+        len(e), firm.sum(), np.median(e), e[firm].max() if firm.any() else 0.0, e.max())
+    ok = e.max() < (TOL[dtype] if dtype == "float32" else 2.0)
+    ok = ok and (not firm.any() or e[firm].max() < TOL[dtype])
+    if len(e) >= 8:
+        ok = ok and np.median(e) < TOL_MEDIAN[dtype]
+    return Verdict(bool(ok), text)
+
+
+def tokens_for(cfg, n, seed):
+    return np.random.default_rng(seed).integers(0, cfg["vocab"], n).tolist()
+
+
+def run_alone(rp, rid, toks, cuts):
+    """Feed `toks` in portions of the sizes `cuts` (the last size repeats); all logits."""
+    out, lo, i = [], 0, 0
+    while lo < len(toks):
+        n = cuts[min(i, len(cuts) - 1)]
+        i += 1
+        hi = min(len(toks), lo + n)
+        lg = rp.step([{"id": rid, "tokens": toks[lo:hi], "want": list(range(hi - lo))}],
+                     [rid] if hi == len(toks) else [])
+        out.append(lg.cpu().numpy())
+        lo = hi
+    return np.concatenate(out)
+
+
+# ---------------------------------------------------------------- whole prompts, decode, portions
+@pytest.mark.parametrize("device,dtype", DEVICES)
+@pytest.mark.parametrize("name", ["mixed", "plain", "wide", "odd"])
+def test_whole_prompt_matches_oracle(models, name, device, dtype):
+    _, cfg, wts = models[name]
+    eng = engine(models, name, device, dtype)
+    rp = TraceReplayer(eng)
+    toks = tokens_for(cfg, 150 if name == "wide" else 61, 1)
+    want = expected(cfg, wts, toks)
+    got = run_alone(rp, "w", toks, [len(toks)])
+    assert close(got, want, dtype)
+    # the first tokens of a sequence, and a one-token prompt
+    assert close(got[:3], want[:3], dtype)
+    one = run_alone(rp, "o", toks[:1], [1])
+    assert close(one, want[:1], dtype)
+
+
+@pytest.mark.parametrize("device,dtype", DEVICES)
+@pytest.mark.parametrize("name", ["mixed", "plain", "wide", "odd"])
+def test_prefill_then_token_by_token(models, name, device, dtype):
+    _, cfg, wts = models[name]
+    eng = engine(models, name, device, dtype)
+    rp = TraceReplayer(eng)
+    toks = tokens_for(cfg, 130 if name == "wide" else 70, 2)
+    want = expected(cfg, wts, toks)
+    if name == "wide":                             # portions across 64-row blocks and key tiles
+        assert close(run_alone(rp, "c", toks, [70, 3, 45, 2, 1]), want, dtype)
+    got = run_alone(rp, "d", toks, [20, 1])
+    assert close(got, want, dtype)
+    got = run_alone(rp, "e", toks, [1])            # decoding from the very first token
+    assert close(got, want, dtype)
+
+
+@pytest.mark.parametrize("device,dtype", DEVICES)
+@pytest.mark.parametrize("cuts", [[2], [3, 2, 7, 2, 11, 5, 1], [8], [9, 16, 2, 1], [1, 2, 1, 3]])
+def test_portions(models, device, dtype, cuts):
+    """Portions down to two tokens (shorter than the convolutions' taps - 1, so a portion's
+    convolution state keeps inputs of the portion before it) and cut inside pages."""
+    _, cfg, wts = models["mixed"]
+    eng = engine(models, "mixed", device, dtype)
+    rp = TraceReplayer(eng)
+    toks = tokens_for(cfg, 45, 3)
+    want = expected(cfg, wts, toks)
+    assert close(run_alone(rp, "p", toks, cuts), want, dtype)
+    _, cfg, wts = models["odd"]                     # five taps: four inputs of state
+    rp = TraceReplayer(engine(models, "odd", device, dtype))
+    toks = tokens_for(cfg, 31, 7)
+    assert close(run_alone(rp, "q", toks, cuts), expected(cfg, wts, toks), dtype)
+
+
+@pytest.mark.parametrize("device,dtype", DEVICES)
+def test_long_decode(models, device, dtype):
+    _, cfg, wts = models["plain"]
+    eng = engine(models, "plain", device, dtype, pages=40)
+    rp = TraceReplayer(eng)
+    toks = tokens_for(cfg, 150, 4)
+    want = expected(cfg, wts, toks)
+    got = run_alone(rp, "l", toks, [5, 1])
+    assert close(got[-20:], want[-20:], dtype)
+    assert close(got, want, dtype)
+
+
+@pytest.mark.parametrize("device,dtype", DEVICES)
+def test_long_prompt(models, device, dtype):
+    """A prompt of several hundred tokens in one step (many row blocks of the convolution
+    and many staged token blocks of the scans), then a second portion and decoded tokens
+    that continue its state."""
+    _, cfg, wts = models["plain"]
+    eng = engine(models, "plain", device, dtype, pages=60)
+    rp = TraceReplayer(eng)
+    toks = tokens_for(cfg, 440, 6)
+    want = expected(cfg, wts, toks)
+    got = run_alone(rp, "L", toks, [300, 130, 1])
+    assert close(got[-40:], want[-40:], dtype)
+    assert close(got, want, dtype)
+
+
+# ---------------------------------------------------------------- batches, pages and slots reused
+@pytest.mark.parametrize("device,dtype", DEVICES)
+@pytest.mark.parametrize("name", ["mixed", "wide"])
+def test_mixed_batches_and_reuse(models, name, device, dtype):
+    """Four live requests of unequal length, portions beside decode rows, requests that
+    sit out steps; the pool (14 pages) and the four slots are used again by later
+    requests.  Every row must match the request run alone (the oracle)."""
+    _, cfg, wts = models[name]
+    eng = engine(models, name, device, dtype, pages=14)
+    rp = TraceReplayer(eng)
+    lens = {"a": 30, "b": 9, "c": 41, "d": 2, "e": 25, "f": 17, "g": 33}
+    toks = {k: tokens_for(cfg, n, 10 + i) for i, (k, n) in enumerate(lens.items())}
+    want = {k: expected(cfg, wts, v) for k, v in toks.items()}
+    at = {k: 0 for k in lens}
+    got = {k: [] for k in lens}
+    # (request, tokens) per step; a request is freed when its tokens are used up
+    plan = [[("a", 7), ("b", 3)], [("a", 1), ("b", 1), ("c", 12)], [("a", 1), ("c", 2), ("d", 2)],
+            [("b", 5), ("c", 1), ("a", 9)], [("a", 1), ("c", 1)], [("a", 11), ("c", 25), ("e", 4)],
+            [("e", 1), ("f", 17)], [("e", 1), ("g", 8)], [("e", 19), ("g", 1)], [("g", 24)]]
+    used_pages = []
+    for step in plan:
+        entries, end = [], []
+        for k, n in step:
+            lo = at[k]
+            entries.append({"id": k, "tokens": toks[k][lo:lo + n], "want": list(range(n))})
+            at[k] += n
+            if at[k] == lens[k]:
+                end.append(k)
+        assert len(rp.seqs) <= 4
+        lg = rp.step(entries, end).cpu().numpy()
+        for s in rp.seqs.values():
+            used_pages += s.block_ids
+        o = 0
+        for k, n in step:
+            got[k].append(lg[o:o + n])
+            o += n
+    assert all(at[k] == lens[k] for k in lens)
+    assert len(used_pages) > len(set(used_pages)) and len(set(used_pages)) <= 14
+    for k in lens:
+        assert close(np.concatenate(got[k]), want[k], dtype), k
+
+
+@pytest.mark.parametrize("device,dtype", DEVICES)
+def test_slot_reuse_starts_from_zero_state(models, device, dtype):
+    """A slot that held a long request is given to a new one: its convolution inputs,
+    recurrent state and pages must not leak into the new request's first tokens."""
+    _, cfg, wts = models["mixed"]
+    eng = engine(models, "mixed", device, dtype, seqs=1, pages=10)
+    rp = TraceReplayer(eng)
+    first, second = tokens_for(cfg, 50, 20), tokens_for(cfg, 12, 21)
+    run_alone(rp, "x", first, [50])
+    got = run_alone(rp, "y", second, [2, 1])
+    assert close(got, expected(cfg, wts, second), dtype)
+
+
+# ---------------------------------------------------------------- residual stream per layer run
+@pytest.mark.parametrize("device,dtype", DEVICES)
+@pytest.mark.parametrize("name", ["mixed", "plain", "odd"])
+def test_layer_taps(models, name, device, dtype):
+    d, cfg, wts = models[name]
+    eng = engine(models, name, device, dtype)
+    runner = eng.executor.runner
+    toks = tokens_for(cfg, 19, 5)
+    want = []
+    oracle.forward(cfg, wts, toks, want)
+    assert len(want) == len(oracle.layer_runs(cfg))
+    rp = TraceReplayer(eng)
+    taps = []
+    model = runner.model
+    orig = model.forward
+    model.forward = lambda *a, **k: orig(*a, taps=taps, **k)
+    try:
+        run_alone(rp, "t", toks, [len(toks)])
+    finally:
+        model.forward = orig
+    assert len(taps) == len(want)
+    tol = 2e-4 if dtype == "float32" else 0.05
+    for got, w in zip(taps, want):
+        g = got.cpu().double().numpy()
+        assert np.abs(g - w).max() <= tol * np.abs(w).max()
+
+
+# ---------------------------------------------------------------- generation entry points
+@pytest.mark.parametrize("device,dtype", DEVICES)
+def test_greedy_generation_through_scheduler(models, device, dtype):
+    """LLM.generate (request intake, continuous batching, chunked prefill with a token
+    budget smaller than the prompts, sampling at temperature 0): every generated token is
+    the oracle's argmax given the tokens before it."""
+    d, cfg, wts = models["mixed"]
+    if device == "cuda" and not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    llm = LLM(model=d, dtype=dtype, device=device, block_size=8, max_num_seqs=3,
+              max_model_len=96, max_num_batched_tokens=16, num_gpu_blocks_override=40,
+              cuda_graph_max_bs=3)
+    try:
+        prompts = [tokens_for(cfg, n, 30 + n) for n in (5, 23, 1, 37, 12)]
+        outs = llm.generate(prompts, SamplingParams(temperature=0.0, max_tokens=12, ignore_eos=True))
+    finally:
+        llm.shutdown()
+    margin = 1e-3 if dtype == "float32" else 0.15
+    for p, o in zip(prompts, outs):
+        gen = list(o.output_token_ids)
+        assert len(gen) == 12
+        lg = oracle.forward(cfg, wts, p + gen)
+        for i, tok in enumerate(gen):
+            row = lg[len(p) - 1 + i]
+            assert row[tok] >= row.max() - margin * (row.max() - row.min()), (i, tok)
+
+
+@pytest.mark.parametrize("device,dtype", [CPU, GPU16])
+def test_preset_with_random_weights_generates(device, dtype):
+    """The built-in small preset with random weights through request intake, the scheduler
+    and sampling (temperature > 0, top-k): the right number of tokens, all in range, and
+    the same tokens again for the same seeds."""
+    if device == "cuda" and not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    outs = []
+    for _ in range(2):
+        llm = LLM(model="tiny-nolesun", dtype=dtype, device=device, random_init=True, seed=3,
+                  block_size=16, max_num_seqs=4, max_model_len=128, max_num_batched_tokens=64,
+                  num_gpu_blocks_override=40, cuda_graph_max_bs=4)
+        try:
+            prompts = [list(range(5, 5 + n)) for n in (3, 40, 17)]
+            res = llm.generate(prompts, SamplingParams(temperature=0.8, top_k=20, max_tokens=9,
+                                                       ignore_eos=True, seed=11))
+        finally:
+            llm.shutdown()
+        outs.append([list(o.output_token_ids) for o in res])
+    assert all(len(o) == 9 and all(0 <= t < 1024 for t in o) for o in outs[0])
+    assert outs[0] == outs[1]
+
+
+def test_registry_and_config_reader(models):
+    from kubernetes_gpu_cluster_amd.models import resolve_model
+    d, cfg, _ = models["mixed"]
+    mc, wdir = resolve_model(d)
+    assert mc.arch == "nolesun" and wdir == d and mc.num_layers == 4
+    assert [s.kind for s in mc.layer_specs] == ["parallel"] * 4
+    assert [s.right.kind for s in mc.layer_specs] == ["mamba2", "gated_delta", "mamba2", "gated_delta"]
+    assert mc.layer_loop == (1, 3, 2) and mc.loop_mix and mc.embed_scale == 3.0
+    sp = mc.layer_specs[1]
+    l, r = sp.left, sp.right
+    assert (l.heads, l.kv_heads, l.dim, l.vdim, l.rot_dims) == (4, 2, 12, 10, 8)
+    assert l.bias and l.elem_gate and l.softcap == 4.0 and l.rotary.interleaved
+    assert (r.heads, r.kv_heads, r.dim, r.vdim, r.conv) == (4, 2, 10, 6, 4)
+    assert (sp.left_scale, sp.right_scale) == (0.7, 1.3)
+    assert (sp.mlp.kind, sp.mlp.experts, sp.mlp.top, sp.mlp.router) == ("moe", 6, 2, "softmax")
+    sp = mc.layer_specs[2]
+    l, r = sp.left, sp.right
+    assert not l.bias and not l.elem_gate and l.softcap == 0.0 and not l.rotary.interleaved
+    assert (r.heads, r.vdim, r.dim, r.kv_heads, r.conv, r.inner_norm_groups) == (2, 12, 6, 1, 2, 1)
+    assert mc.layer_specs[0].mlp.kind == "dense" and not mc.layer_specs[0].mlp.gated
+    assert mc.layer_specs[3].mlp is None and mc.has_recurrent_state
+    mp, _ = resolve_model(models["plain"][0])
+    assert mp.layer_loop is None and not mp.loop_mix and mp.embed_scale == 1.0
