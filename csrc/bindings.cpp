@@ -1377,7 +1377,8 @@ int64_t table_stride(const std::optional<Tensor>& bt, int64_t rows, int64_t othe
   if (!bt.has_value() || rows == 0) return other;
   TORCH_CHECK(bt->dim() == 2 && bt->size(0) >= rows && bt->stride(1) == 1,
               "kgc: block tables [rows, max_blocks]");
-  return bt->stride(0);
+  // a single row may carry any stride; the kernels also take the stride as the row's length
+  return bt->size(0) == 1 ? bt->size(1) : bt->stride(0);
 }
 
 void window_attention(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
