@@ -1,5 +1,6 @@
 """Microbenchmarks of the hybrid-decoder kernels beside the Llama-path kernel each one is
-closest to, at the layer shapes of the dilavik-w2048 / konovik-w2048 / llama-w2048 presets.
+closest to, at the layer shapes of the dilavik-w2048 / konovik-w2048 / nolesun-w2048 /
+llama-w2048 presets (``--only nolesun``: the parallel mixers' kernels).
 
     python tools/hybrid_bench.py [--reps 20] > profiles/hybrid_kernels.jsonl
 
@@ -287,6 +288,78 @@ def konovik(reps):
         emit("side_gate", f"{T}x64", us, gbytes=T * 64 * 6 / 1e9)
 
 
+def nolesun(reps):
+    """The parallel mixers' kernels at the nolesun-w2048 layer shapes: the causal convolution,
+    both scans, the gated norms, and the attention with capped scores writing a column slice."""
+    W = 2048
+    shapes = (("prefill 32x512", [512] * 32, []), ("prefill 2x8192", [8192] * 2, []),
+              ("decode 64", [], [544] * 64), ("decode 256", [], [544] * 256))
+    for name, P_q, D_ctx in shapes:
+        n = len(P_q) + len(D_ctx)
+        m, _, _ = meta(P_q, list(P_q), D_ctx, 32, DEV, slots=list(range(n)))
+        T = sum(P_q) + len(D_ctx)
+        # Mamba-2: 32 heads of 64, state 128, one group, 4 taps
+        H, V, N, G, K = 32, 64, 128, 1, 4
+        C = H * V + 2 * G * N
+        proj = torch.randn(T, 2 * H * V + 2 * G * N + H, device=DEV, dtype=BF)
+        cw, cb = torch.randn(C, K, device=DEV) * 0.3, torch.randn(C, device=DEV) * 0.1
+        cst = torch.zeros(n, K - 1, C, device=DEV)
+        us = timed(lambda: ops.causal_conv(proj[:, H * V: H * V + C], cw, cb, cst, m), reps)
+        emit("causal_conv (x | B | C, 4 taps)", name, us, gbytes=T * C * 6 / 1e9, like="token_shift")
+        xbc = torch.randn(T, C, device=DEV)
+        par = (torch.rand(H, device=DEV), torch.randn(H, device=DEV) - 2, torch.ones(H, device=DEV))
+        S = torch.zeros(n, H, N, V, device=DEV)
+        us = timed(lambda: ops.ssd_scan(xbc, proj[:, -H:], *par, S, m, H, V, N, G), reps)
+        emit("ssd_scan", name, us, gbytes=2 * n * H * N * V * 4 / 1e9, tflop=4 * T * H * N * V / 1e12,
+             like="mlstm_scan")
+        y = torch.randn(T, H * V, device=DEV)
+        feats = torch.empty(T, 2 * W, device=DEV, dtype=BF)
+        nw = torch.ones(H * V, device=DEV)
+        us = timed(lambda: ops.gated_rms_norm(y, proj[:, : H * V], nw, 1, 1e-6, True, feats[:, W:]), reps)
+        emit("gated_rms_norm (gate, then norm of the row)", f"{T}x{H * V}", us,
+             gbytes=T * H * V * 8 / 1e9, like="head_norm_gate")
+        # gated delta rule: 16 heads of 128 x 128 over 8 query / key heads, 4 taps
+        H, G, d, V = 16, 8, 128, 128
+        C = 2 * G * d + H * V
+        proj = torch.randn(T, C + H * V + 2 * H, device=DEV, dtype=BF)
+        cw = torch.randn(C, K, device=DEV) * 0.3
+        cst = torch.zeros(n, K - 1, C, device=DEV)
+        us = timed(lambda: ops.causal_conv(proj[:, :C], cw, None, cst, m), reps)
+        emit("causal_conv (q | k | v, 4 taps)", name, us, gbytes=T * C * 6 / 1e9, like="token_shift")
+        qkv = torch.randn(T, C, device=DEV)
+        S = torch.zeros(n, H, d, V, device=DEV)
+        us = timed(lambda: ops.gated_delta_scan(qkv, proj[:, -2 * H:], par[0][:H], par[1][:H], S, m,
+                                                H, G, d, V), reps)
+        emit("gated_delta_scan", name, us, gbytes=2 * n * H * d * V * 4 / 1e9,
+             tflop=6 * T * H * d * V / 1e12, like="mlstm_scan")
+        o = torch.randn(T, H * V, device=DEV)
+        nw = torch.ones(H * V, device=DEV)
+        us = timed(lambda: ops.gated_rms_norm(o, proj[:, C: C + H * V], nw, H, 1e-6, False,
+                                              feats[:, W:]), reps)
+        emit("gated_rms_norm (norm per head, then gate)", f"{T}x{H * V}", us,
+             gbytes=T * H * V * 8 / 1e9, like="head_norm_gate")
+    # attention: plain causal with a score cap, into a column slice, beside the windowed kernel
+    H, G, d, bs = 16, 4, 128, 32
+    for name, P_q, P_sl, D_ctx in (("prefill 32x512", [512] * 32, [512] * 32, []),
+                                   ("prefill 8x2048", [2048] * 8, [2048] * 8, []),
+                                   ("decode 64 @544", [], [], [544] * 64),
+                                   ("decode 256 @544", [], [], [544] * 256)):
+        m, tables, nb = meta(P_q, P_sl, D_ctx, bs, DEV)
+        T = sum(P_q) + len(D_ctx)
+        q = torch.randn(T, H, d, device=DEV, dtype=BF)
+        kc = torch.randn(nb, G, bs, d, device=DEV, dtype=BF)
+        vc = torch.randn(nb, G, bs, d, device=DEV, dtype=BF)
+        pos = torch.zeros(T, dtype=torch.int64, device=DEV)
+        feats = torch.empty(T, 2 * H * d, device=DEV, dtype=BF)
+        keys = sum(s * (s + 1) // 2 for s in P_sl) if P_q else sum(D_ctx)
+        for cap in (0.0, 30.0):
+            us = timed(lambda: ops.window_attention(q, kc, vc, pos, m, 0.09, 0, 0, None, cap, 1.2,
+                                                    out=feats[:, : H * d]), reps)
+            emit("window_attention (causal%s, into a slice)" % (", capped" if cap else ""), name, us,
+                 gbytes=None if P_q else keys * G * 2 * d * 2 / 1e9,
+                 tflop=keys * H * 4 * d / 1e12 if P_q else None, like="window_attention")
+
+
 if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--reps", type=int, default=20)
@@ -294,4 +367,5 @@ if __name__ == "__main__":
     a = ap.parse_args()
     ops.load_extension(strict=True)
     for part in a.only.split(","):
-        {"attention": attention, "recurrent": recurrent, "rows": rows, "konovik": konovik}[part](a.reps)
+        {"attention": attention, "recurrent": recurrent, "rows": rows, "konovik": konovik,
+         "nolesun": nolesun}[part](a.reps)
