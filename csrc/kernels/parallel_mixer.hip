@@ -12,9 +12,9 @@
 // gives zeros.  Prefill chunks and decode rows run the same code, token by token, so a
 // position's result does not depend on how the prompt was cut.
 //
-// Scan layout: grid (step sequences, heads, ceil(value columns / 64)), 256 threads.  The
-// state of one head is S [R, V] (R: state size N or key size d; V: value columns).  A wave
-// owns 16 columns; its lanes are (row group rg = lane / 16, column lane % 16) and a lane
+// Scan layout: grid (step sequences, heads, value-column tiles), four waves.  The state of
+// one head is S [R, V] (R: state size N or key size d; V: value columns).  A wave owns 16
+// columns (4 when few long sequences have to cover the chip: see scan_narrow); its lanes are (row group rg = lane / 16, column lane % 16) and a lane
 // keeps rows rg, rg + 4, rg + 8, ... of its column in registers for the whole chunk, so S
 // is read and written once per step and a token's sums over rows end with two cross-lane
 // steps inside the wave: no barrier per token.  Tokens are staged in LDS 16 at a time.
@@ -106,16 +106,24 @@ __global__ __launch_bounds__(NT) void causal_conv_kernel(
     old[j] = v;
   }
   const float b = bias != nullptr ? bias[c] : 0.f;
-  for (int r = 0; r < nrows; ++r) {
-    const float cur = to_f(xc[(int64_t)(r0 + r) * xs]);
-    float acc = b;
+  constexpr int RB = 8;                    // rows whose loads are in flight together
+  for (int rb = 0; rb < nrows; rb += RB) {
+    float in[RB];
 #pragma unroll
-    for (int j = 0; j < K - 1; ++j) acc += wk[j] * win[j];
-    acc += wk[K - 1] * cur;
+    for (int u = 0; u < RB; ++u)
+      in[u] = rb + u < nrows ? to_f(xc[(int64_t)(r0 + rb + u) * xs]) : 0.f;
 #pragma unroll
-    for (int j = 0; j + 1 < K - 1; ++j) win[j] = win[j + 1];
-    if constexpr (K > 1) win[K - 2] = cur;
-    orow[(int64_t)r * C] = silu ? acc * sigmoid_f(acc) : acc;
+    for (int u = 0; u < RB; ++u) {
+      const float cur = in[u];
+      float acc = b;
+#pragma unroll
+      for (int j = 0; j < K - 1; ++j) acc += wk[j] * win[j];
+      acc += wk[K - 1] * cur;
+#pragma unroll
+      for (int j = 0; j + 1 < K - 1; ++j) win[j] = win[j + 1];
+      if constexpr (K > 1) win[K - 2] = cur;
+      if (rb + u < nrows) orow[(int64_t)(rb + u) * C] = silu ? acc * sigmoid_f(acc) : acc;
+    }
   }
   if (r0 == 0) {
     // the chunk's last K - 1 inputs; a chunk shorter than that keeps some of the old ones
@@ -138,23 +146,24 @@ __global__ __launch_bounds__(NT) void causal_conv_kernel(
 
 // ---- Mamba-2 recurrence ---------------------------------------------------------------------
 // xbc fp32 [T, H V + 2 G N] = x | B | C; dt [T, H] (row stride dts) raw step sizes.
-// RPT: rows of S per lane (N <= 4 RPT).
-template <typename T, int RPT>
+// RPT: rows of S per lane (N <= row groups * RPT); LOGC: log2 of the columns per wave.
+template <typename T, int RPT, int LOGC>
 __global__ __launch_bounds__(NT) void ssd_scan_kernel(
     float* __restrict__ out, const float* __restrict__ xbc, const T* __restrict__ dt,
     int64_t dts, const float* __restrict__ a_log, const float* __restrict__ dt_bias,
     const float* __restrict__ dskip, float* __restrict__ S, const int* __restrict__ qsl,
     const int* __restrict__ seq_lens, const int* __restrict__ ctx_lens,
     const int* __restrict__ slots, int P, int Tp, int H, int V, int N, int G, int num_slots) {
-  constexpr int RP = 4 * RPT;
+  constexpr int CW = 1 << LOGC, NRG = 64 >> LOGC;     // columns per wave, row groups per wave
+  constexpr int RP = NRG * RPT, NTH = NT, CT = CW * (NT / 64);   // rows (padded), threads, columns per workgroup
   extern __shared__ float lds[];
   float* Bs = lds;                   // [TB][RP]
   float* Cs = Bs + TB * RP;          // [TB][RP]
-  float* xv = Cs + TB * RP;          // [TB][64]
-  float* sc = xv + TB * 64;          // [TB][2]: decay, step size
+  float* xv = Cs + TB * RP;          // [TB][CT]
+  float* sc = xv + TB * CT;          // [TB][2]: decay, step size
   const int s = blockIdx.x, h = blockIdx.y;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, rg = lane >> 4;
-  const int lc = wave * 16 + (lane & 15), col = blockIdx.z * 64 + lc;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, rg = lane >> LOGC;
+  const int lc = wave * CW + (lane & (CW - 1)), col = blockIdx.z * CT + lc;
   const bool colok = col < V;
   const StepSeq q = step_seq(s, P, Tp, qsl, seq_lens, ctx_lens, slots);
   const int64_t ow = (int64_t)H * V;
@@ -171,13 +180,13 @@ __global__ __launch_bounds__(NT) void ssd_scan_kernel(
   float Sr[RPT];
 #pragma unroll
   for (int i = 0; i < RPT; ++i) {
-    const int r = 4 * i + rg;
+    const int r = NRG * i + rg;
     Sr[i] = (!fresh && r < N && colok) ? Sp[(int64_t)r * V + col] : 0.f;
   }
   const float A = expf(a_log[h]), dtb = dt_bias[h], Dh = dskip[h];
   for (int t0 = 0; t0 < q.len; t0 += TB) {
     const int nb = min(TB, q.len - t0);
-    for (int e = threadIdx.x; e < TB * RP; e += NT) {
+    for (int e = threadIdx.x; e < TB * RP; e += NTH) {
       const int tb = e / RP, r = e - tb * RP;
       float bv = 0.f, cv = 0.f;
       if (tb < nb && r < N) {
@@ -188,8 +197,8 @@ __global__ __launch_bounds__(NT) void ssd_scan_kernel(
       Bs[e] = bv;
       Cs[e] = cv;
     }
-    for (int e = threadIdx.x; e < TB * 64; e += NT) {
-      const int tb = e >> 6, c = blockIdx.z * 64 + (e & 63);
+    for (int e = threadIdx.x; e < TB * CT; e += NTH) {
+      const int tb = e / CT, c = blockIdx.z * CT + (e - tb * CT);
       xv[e] = (tb < nb && c < V) ? xbc[(int64_t)(q.start + t0 + tb) * cw + xoff + c] : 0.f;
     }
     if (threadIdx.x < TB) {
@@ -205,24 +214,24 @@ __global__ __launch_bounds__(NT) void ssd_scan_kernel(
     __syncthreads();
     for (int tb = 0; tb < nb; ++tb) {
       const float a = sc[2 * tb], d = sc[2 * tb + 1];
-      const float xc = xv[tb * 64 + lc], xd = d * xc;
+      const float xc = xv[tb * CT + lc], xd = d * xc;
       const float* bp = Bs + tb * RP + rg;
       const float* cp = Cs + tb * RP + rg;
       float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;       // independent chains
 #pragma unroll
       for (int i = 0; i < RPT; i += 4) {
-        Sr[i] = a * Sr[i] + bp[4 * i] * xd;
-        Sr[i + 1] = a * Sr[i + 1] + bp[4 * i + 4] * xd;
-        Sr[i + 2] = a * Sr[i + 2] + bp[4 * i + 8] * xd;
-        Sr[i + 3] = a * Sr[i + 3] + bp[4 * i + 12] * xd;
-        a0 += Sr[i] * cp[4 * i];
-        a1 += Sr[i + 1] * cp[4 * i + 4];
-        a2 += Sr[i + 2] * cp[4 * i + 8];
-        a3 += Sr[i + 3] * cp[4 * i + 12];
+        Sr[i] = a * Sr[i] + bp[NRG * i] * xd;
+        Sr[i + 1] = a * Sr[i + 1] + bp[NRG * (i + 1)] * xd;
+        Sr[i + 2] = a * Sr[i + 2] + bp[NRG * (i + 2)] * xd;
+        Sr[i + 3] = a * Sr[i + 3] + bp[NRG * (i + 3)] * xd;
+        a0 += Sr[i] * cp[NRG * i];
+        a1 += Sr[i + 1] * cp[NRG * (i + 1)];
+        a2 += Sr[i + 2] * cp[NRG * (i + 2)];
+        a3 += Sr[i + 3] * cp[NRG * (i + 3)];
       }
       float y = (a0 + a1) + (a2 + a3);
-      y += __shfl_xor(y, 16, 64);
-      y += __shfl_xor(y, 32, 64);
+#pragma unroll
+      for (int o = CW; o < 64; o <<= 1) y += __shfl_xor(y, o, 64);
       if (rg == 0 && colok)
         out[(int64_t)(q.start + t0 + tb) * ow + h * V + col] = y + Dh * xc;
     }
@@ -230,7 +239,7 @@ __global__ __launch_bounds__(NT) void ssd_scan_kernel(
   }
 #pragma unroll
   for (int i = 0; i < RPT; ++i) {
-    const int r = 4 * i + rg;
+    const int r = NRG * i + rg;
     if (r < N && colok) Sp[(int64_t)r * V + col] = Sr[i];
   }
 }
@@ -240,22 +249,23 @@ __global__ __launch_bounds__(NT) void ssd_scan_kernel(
 // pre-activations.  With the token's S_0 = the state before it:
 //   S^T k = g S_0^T k,  o = S_new^T q = g S_0^T q + (k . q) u,  S_new = g S_0 + k u^T
 // so both sums over rows are taken over S_0 in one pass.
-template <typename T, int RPT>
+template <typename T, int RPT, int LOGC>
 __global__ __launch_bounds__(NT) void gated_delta_scan_kernel(
     float* __restrict__ out, const float* __restrict__ qkv, const T* __restrict__ ba,
     int64_t bas, const float* __restrict__ a_log, const float* __restrict__ dt_bias,
     float* __restrict__ S, const int* __restrict__ qsl, const int* __restrict__ seq_lens,
     const int* __restrict__ ctx_lens, const int* __restrict__ slots, int P, int Tp, int H,
     int G, int d, int V, int num_slots) {
-  constexpr int RP = 4 * RPT;
+  constexpr int CW = 1 << LOGC, NRG = 64 >> LOGC;     // columns per wave, row groups per wave
+  constexpr int RP = NRG * RPT, NTH = NT, CT = CW * (NT / 64);   // rows (padded), threads, columns per workgroup
   extern __shared__ float lds[];
   float* ks = lds;                   // [TB][RP]
   float* qs = ks + TB * RP;          // [TB][RP]
-  float* vs = qs + TB * RP;          // [TB][64]
-  float* sc = vs + TB * 64;          // [TB][3]: decay, write strength, k . q
+  float* vs = qs + TB * RP;          // [TB][CT]
+  float* sc = vs + TB * CT;          // [TB][3]: decay, write strength, k . q
   const int s = blockIdx.x, h = blockIdx.y;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, rg = lane >> 4;
-  const int lc = wave * 16 + (lane & 15), col = blockIdx.z * 64 + lc;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, rg = lane >> LOGC;
+  const int lc = wave * CW + (lane & (CW - 1)), col = blockIdx.z * CT + lc;
   const bool colok = col < V;
   const StepSeq q = step_seq(s, P, Tp, qsl, seq_lens, ctx_lens, slots);
   const int64_t ow = (int64_t)H * V;
@@ -272,13 +282,13 @@ __global__ __launch_bounds__(NT) void gated_delta_scan_kernel(
   float Sr[RPT];
 #pragma unroll
   for (int i = 0; i < RPT; ++i) {
-    const int r = 4 * i + rg;
+    const int r = NRG * i + rg;
     Sr[i] = (!fresh && r < d && colok) ? Sp[(int64_t)r * V + col] : 0.f;
   }
   const float A = expf(a_log[h]), dtb = dt_bias[h], qscale = 1.f / sqrtf((float)d);
   for (int t0 = 0; t0 < q.len; t0 += TB) {
     const int nb = min(TB, q.len - t0);
-    for (int e = threadIdx.x; e < TB * RP; e += NT) {
+    for (int e = threadIdx.x; e < TB * RP; e += NTH) {
       const int tb = e / RP, r = e - tb * RP;
       float kv = 0.f, qv = 0.f;
       if (tb < nb && r < d) {
@@ -289,8 +299,8 @@ __global__ __launch_bounds__(NT) void gated_delta_scan_kernel(
       ks[e] = kv;
       qs[e] = qv;
     }
-    for (int e = threadIdx.x; e < TB * 64; e += NT) {
-      const int tb = e >> 6, c = blockIdx.z * 64 + (e & 63);
+    for (int e = threadIdx.x; e < TB * CT; e += NTH) {
+      const int tb = e / CT, c = blockIdx.z * CT + (e - tb * CT);
       vs[e] = (tb < nb && c < V) ? qkv[(int64_t)(q.start + t0 + tb) * cw + voff + c] : 0.f;
     }
     __syncthreads();
@@ -321,25 +331,26 @@ __global__ __launch_bounds__(NT) void gated_delta_scan_kernel(
     __syncthreads();
     for (int tb = 0; tb < nb; ++tb) {
       const float gd = sc[3 * tb], beta = sc[3 * tb + 1], kq = sc[3 * tb + 2];
-      const float vv = vs[tb * 64 + lc];
+      const float vv = vs[tb * CT + lc];
       const float* kp = ks + tb * RP + rg;
       const float* qp = qs + tb * RP + rg;
       float k0 = 0.f, k1 = 0.f, q0 = 0.f, q1 = 0.f;
 #pragma unroll
       for (int i = 0; i < RPT; i += 2) {
-        k0 += Sr[i] * kp[4 * i];
-        k1 += Sr[i + 1] * kp[4 * i + 4];
-        q0 += Sr[i] * qp[4 * i];
-        q1 += Sr[i + 1] * qp[4 * i + 4];
+        k0 += Sr[i] * kp[NRG * i];
+        k1 += Sr[i + 1] * kp[NRG * (i + 1)];
+        q0 += Sr[i] * qp[NRG * i];
+        q1 += Sr[i + 1] * qp[NRG * (i + 1)];
       }
       float sk = k0 + k1, sq = q0 + q1;
-      sk += __shfl_xor(sk, 16, 64);
-      sq += __shfl_xor(sq, 16, 64);
-      sk += __shfl_xor(sk, 32, 64);
-      sq += __shfl_xor(sq, 32, 64);
+#pragma unroll
+      for (int o = CW; o < 64; o <<= 1) {
+        sk += __shfl_xor(sk, o, 64);
+        sq += __shfl_xor(sq, o, 64);
+      }
       const float u = beta * (vv - gd * sk);
 #pragma unroll
-      for (int i = 0; i < RPT; ++i) Sr[i] = gd * Sr[i] + kp[4 * i] * u;
+      for (int i = 0; i < RPT; ++i) Sr[i] = gd * Sr[i] + kp[NRG * i] * u;
       if (rg == 0 && colok)
         out[(int64_t)(q.start + t0 + tb) * ow + h * V + col] = gd * sq + kq * u;
     }
@@ -347,7 +358,7 @@ __global__ __launch_bounds__(NT) void gated_delta_scan_kernel(
   }
 #pragma unroll
   for (int i = 0; i < RPT; ++i) {
-    const int r = 4 * i + rg;
+    const int r = NRG * i + rg;
     if (r < d && colok) Sp[(int64_t)r * V + col] = Sr[i];
   }
 }
@@ -429,8 +440,21 @@ void launch_causal_conv(int dtype, float* out, const void* x, int64_t xs, const 
 
 int matrix_scan_max_rows() { return 256; }
 
-static size_t scan_lds(int rpt, int extra) {
-  return sizeof(float) * (size_t)(2 * TB * 4 * rpt + TB * 64 + TB * extra);
+static size_t scan_lds(int rows_padded, int cols, int extra) {
+  return sizeof(float) * (size_t)(2 * TB * rows_padded + TB * cols + TB * extra);
+}
+
+// columns per wave: 16 (a lane holds every 4th row of its column) when that already gives the
+// chip two workgroups per CU, else 4 (every 16th row: a quarter of the work per wave and two
+// more cross-lane steps per sum), so that few long sequences still spread over the chip
+static bool scan_narrow(int seqs, int H, int V) {
+  return V <= 4 || (int64_t)seqs * H * ((V + 63) / 64) < 512;
+}
+
+static int pow2_at_least(int n, int lo) {
+  int p = lo;
+  while (p < n) p <<= 1;
+  return p;
 }
 
 void launch_ssd_scan(int dtype, float* out, const float* xbc, const void* dt, int64_t dts,
@@ -439,17 +463,26 @@ void launch_ssd_scan(int dtype, float* out, const float* xbc, const void* dt, in
                      int P, int D, int Tp, int H, int V, int N, int G, int num_slots,
                      hipStream_t s) {
   if (P + D <= 0) return;
-  const dim3 grid(P + D, H, (V + 63) / 64);
-#define KGC_SSD(R)                                                                           \
-  KGC_PM_DISPATCH_T(dtype, ssd_scan_kernel<T, R><<<grid, NT, scan_lds(R, 2), s>>>(           \
+  const bool narrow = scan_narrow(P + D, H, V);
+  const int ct = narrow ? 16 : 64, rp = pow2_at_least(N, narrow ? 64 : 16);
+  const dim3 grid(P + D, H, (V + ct - 1) / ct);
+#define KGC_SSD_W(R, L)                                                                      \
+  KGC_PM_DISPATCH_T(dtype, ssd_scan_kernel<T, R, L><<<grid, NT, scan_lds(rp, ct, 2), s>>>(   \
       out, xbc, (const T*)dt, dts, a_log, dt_bias, dskip, S, qsl, seq_lens, ctx_lens, slots, P, \
       Tp, H, V, N, G, num_slots))
-  if (N <= 16) KGC_SSD(4);
-  else if (N <= 32) KGC_SSD(8);
-  else if (N <= 64) KGC_SSD(16);
-  else if (N <= 128) KGC_SSD(32);
-  else KGC_SSD(64);
-#undef KGC_SSD
+  // rows per lane = padded rows / row groups (4 wide, 16 narrow); at least 4
+  if (!narrow) {
+    if (rp <= 16) KGC_SSD_W(4, 4);
+    else if (rp == 32) KGC_SSD_W(8, 4);
+    else if (rp == 64) KGC_SSD_W(16, 4);
+    else if (rp == 128) KGC_SSD_W(32, 4);
+    else KGC_SSD_W(64, 4);
+  } else {
+    if (rp <= 64) KGC_SSD_W(4, 2);
+    else if (rp == 128) KGC_SSD_W(8, 2);
+    else KGC_SSD_W(16, 2);
+  }
+#undef KGC_SSD_W
 }
 
 void launch_gated_delta_scan(int dtype, float* out, const float* qkv, const void* ba,
@@ -458,17 +491,25 @@ void launch_gated_delta_scan(int dtype, float* out, const float* qkv, const void
                              const int* slots, int P, int D, int Tp, int H, int G, int d, int V,
                              int num_slots, hipStream_t s) {
   if (P + D <= 0) return;
-  const dim3 grid(P + D, H, (V + 63) / 64);
-#define KGC_GD(R)                                                                            \
-  KGC_PM_DISPATCH_T(dtype, gated_delta_scan_kernel<T, R><<<grid, NT, scan_lds(R, 3), s>>>(   \
+  const bool narrow = scan_narrow(P + D, H, V);
+  const int ct = narrow ? 16 : 64, rp = pow2_at_least(d, narrow ? 64 : 16);
+  const dim3 grid(P + D, H, (V + ct - 1) / ct);
+#define KGC_GD_W(R, L)                                                                       \
+  KGC_PM_DISPATCH_T(dtype, gated_delta_scan_kernel<T, R, L><<<grid, NT, scan_lds(rp, ct, 3), s>>>( \
       out, qkv, (const T*)ba, bas, a_log, dt_bias, S, qsl, seq_lens, ctx_lens, slots, P, Tp, H, \
       G, d, V, num_slots))
-  if (d <= 16) KGC_GD(4);
-  else if (d <= 32) KGC_GD(8);
-  else if (d <= 64) KGC_GD(16);
-  else if (d <= 128) KGC_GD(32);
-  else KGC_GD(64);
-#undef KGC_GD
+  if (!narrow) {
+    if (rp <= 16) KGC_GD_W(4, 4);
+    else if (rp == 32) KGC_GD_W(8, 4);
+    else if (rp == 64) KGC_GD_W(16, 4);
+    else if (rp == 128) KGC_GD_W(32, 4);
+    else KGC_GD_W(64, 4);
+  } else {
+    if (rp <= 64) KGC_GD_W(4, 2);
+    else if (rp == 128) KGC_GD_W(8, 2);
+    else KGC_GD_W(16, 2);
+  }
+#undef KGC_GD_W
 }
 
 void launch_gated_rms_norm(int dtype, void* out, int64_t os, const float* y, const void* gate,

@@ -245,6 +245,38 @@ def test_scans_in_a_batch_with_padding_rows(dev):
     assert float(st[1].min()) == 3.0 and float(st[1].max()) == 3.0
 
 
+@pytest.mark.parametrize("dev", DEV)
+def test_scans_with_many_sequences_and_heads(dev):
+    """Sixteen prompts of unequal length and 32 heads in one step: the grid size at which the
+    GPU kernels keep 16 value columns per wave (smaller steps keep 4)."""
+    dev = dev_of(dev)
+    rng = np.random.default_rng(13)
+    lens = [1, 2, 3, 5, 8, 13, 16, 17, 21, 30, 31, 32, 33, 34, 40, 47]
+    T, off = sum(lens), np.concatenate([[0], np.cumsum(lens)])
+    m, _ = meta_for([(0, n) for n in lens], [], None, dev, list(range(16)))
+    H, V, N, G = 32, 24, 20, 4
+    xbc, dt = rng.normal(size=(T, H * V + 2 * G * N)), rng.normal(size=(T, H))
+    a_log, dtb, D = rng.normal(size=H) * 0.5, rng.normal(size=H), rng.normal(size=H)
+    st = torch.full((16, H, N, V), 2.0, device=dev)
+    got = ops.ssd_scan(f32(xbc, dev), f32(dt, dev), f32(a_log, dev), f32(dtb, dev), f32(D, dev), st, m,
+                       H, V, N, G).cpu().numpy()
+    for i in (0, 1, 7, 12, 15):
+        x = xbc[off[i]:off[i + 1]]
+        want = ssd_oracle(x[:, :H * V], x[:, H * V:H * V + G * N], x[:, H * V + G * N:],
+                          dt[off[i]:off[i + 1]], a_log, dtb, D, H, V, N, G)
+        np.testing.assert_allclose(got[off[i]:off[i + 1]], want, rtol=2e-4, atol=2e-4 * np.abs(want).max())
+    H, G, d, V = 32, 8, 20, 24
+    qkv, ba = rng.normal(size=(T, 2 * G * d + H * V)), rng.normal(size=(T, 2 * H))
+    st = torch.full((16, H, d, V), 2.0, device=dev)
+    got = ops.gated_delta_scan(f32(qkv, dev), f32(ba, dev), f32(a_log, dev), f32(dtb, dev), st, m,
+                               H, G, d, V).cpu().numpy()
+    for i in (0, 1, 7, 12, 15):
+        x, b = qkv[off[i]:off[i + 1]], ba[off[i]:off[i + 1]]
+        want = delta_oracle(x[:, :G * d], x[:, G * d:2 * G * d], x[:, 2 * G * d:], b[:, :H], b[:, H:],
+                            a_log, dtb, H, G, d, V)
+        np.testing.assert_allclose(got[off[i]:off[i + 1]], want, rtol=2e-4, atol=2e-4 * np.abs(want).max())
+
+
 # ---------------------------------------------------------------- gated norms
 @pytest.mark.parametrize("dev", DEV)
 @pytest.mark.parametrize("n,groups", [(96, 3), (128, 1), (2048, 2), (66, 6)])
