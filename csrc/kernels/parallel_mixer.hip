@@ -27,7 +27,7 @@ namespace {
 
 constexpr int NT = 256;
 constexpr int TB = 16;             // tokens staged per block
-constexpr int CV_ROWS = 64;        // rows of a chunk per convolution workgroup
+constexpr int CV_ROWS = 32;        // rows of a chunk per convolution workgroup
 constexpr int CV_KMAX = 8;
 
 struct StepSeq {
@@ -57,12 +57,47 @@ __device__ __forceinline__ float softplus_f(float x) {
 __device__ __forceinline__ float sigmoid_f(float x) { return 1.f / (1.f + expf(-x)); }
 
 // ---- causal convolution -------------------------------------------------------------------
-// grid (n_work * (blk_rows / CV_ROWS) + D, ceil(C / 256)): a prefill work item is
+// grid (n_work * (blk_rows / CV_ROWS) + D, channel tiles): a prefill work item is
 // (sequence, block of blk_rows chunk rows), cut into pieces of CV_ROWS rows; one thread walks
-// a channel through its piece with the last K - 1 inputs in registers.  Only the piece that
+// one channel (or four adjacent ones) through its piece with the last K - 1 inputs in
+// registers.  Only the piece that
 // holds a chunk's first row reads the sequence's state (CV_ROWS >= K - 1), and the same
 // thread replaces it afterwards, so no other workgroup touches it meanwhile.
-template <typename T, int K>
+// VEC adjacent channels of one row as fp32 (one 8- or 16-byte load when VEC = 4)
+template <typename T, int VEC>
+__device__ __forceinline__ void load_channels(const T* p, float (&v)[VEC]) {
+  if constexpr (VEC == 1) {
+    v[0] = to_f(p[0]);
+  } else if constexpr (std::is_same_v<T, float>) {
+    const float4 a = *reinterpret_cast<const float4*>(p);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+  } else {
+    Pack4<T> t;
+    t.u = *reinterpret_cast<const u32x2*>(p);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = to_f(t.h[e]);
+  }
+}
+
+template <int VEC>
+__device__ __forceinline__ void load_f32(const float* p, float (&v)[VEC]) {
+  if constexpr (VEC == 1) {
+    v[0] = p[0];
+  } else {
+    const float4 a = *reinterpret_cast<const float4*>(p);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+  }
+}
+
+template <int VEC>
+__device__ __forceinline__ void store_f32(float* p, const float (&v)[VEC]) {
+  if constexpr (VEC == 1) p[0] = v[0];
+  else *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+}
+
+// VEC: adjacent channels per thread (4 where the column slice, the channel count and the
+// row stride allow 8- / 16-byte accesses, else 1)
+template <typename T, int K, int VEC>
 __global__ __launch_bounds__(NT) void causal_conv_kernel(
     float* __restrict__ out, const T* __restrict__ x, int64_t xs, const float* __restrict__ w,
     const float* __restrict__ bias, float* __restrict__ state, const int* __restrict__ qsl,
@@ -70,6 +105,7 @@ __global__ __launch_bounds__(NT) void causal_conv_kernel(
     const int* __restrict__ slots, const int* __restrict__ work_seq,
     const int* __restrict__ work_blk, int n_work, int blk_rows, int P, int Tp, int C,
     int num_slots, bool silu) {
+  constexpr int KS = K > 1 ? K - 1 : 1;      // state rows (arrays of at least one entry)
   const int subs = blk_rows / CV_ROWS;
   const int item = blockIdx.x;
   int s, r0;
@@ -81,48 +117,67 @@ __global__ __launch_bounds__(NT) void causal_conv_kernel(
     r0 = 0;
   }
   const StepSeq q = step_seq(s, P, Tp, qsl, seq_lens, ctx_lens, slots);
-  const int c = blockIdx.y * NT + threadIdx.x;
+  const int c = (blockIdx.y * NT + threadIdx.x) * VEC;
   if (c >= C || r0 >= q.len) return;
   const int nrows = min(CV_ROWS, q.len - r0);
   float* orow = out + (int64_t)(q.start + r0) * C + c;
   if (q.slot < 0 || q.slot >= num_slots || q.pos0 < 0) {
-    for (int r = 0; r < nrows; ++r) orow[(int64_t)r * C] = 0.f;
+    float z[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) z[v] = 0.f;
+    for (int r = 0; r < nrows; ++r) store_f32<VEC>(orow + (int64_t)r * C, z);
     return;
   }
   const bool fresh = q.pos0 == 0;
-  float wk[K], win[K], old[K];
+  float wk[VEC][K], win[KS][VEC], old[KS][VEC], b[VEC];
 #pragma unroll
-  for (int j = 0; j < K; ++j) wk[j] = w[(int64_t)c * K + j];
+  for (int v = 0; v < VEC; ++v) {
+#pragma unroll
+    for (int j = 0; j < K; ++j) wk[v][j] = w[(int64_t)(c + v) * K + j];
+    b[v] = bias != nullptr ? bias[c + v] : 0.f;
+  }
   float* st = state + (int64_t)q.slot * (K - 1) * C + c;
   const T* xc = x + (int64_t)q.start * xs + c;
-  // win[j], j < K - 1: the input at chunk row r0 - (K - 1) + j
+  // win[j], j < K - 1: the inputs at chunk row r0 - (K - 1) + j
 #pragma unroll
   for (int j = 0; j < K - 1; ++j) {
     const int idx = r0 - (K - 1) + j;
-    float v = 0.f;
-    if (idx >= 0) v = to_f(xc[(int64_t)idx * xs]);
-    else if (!fresh) v = st[(int64_t)(K - 1 + idx) * C];
-    win[j] = v;
-    old[j] = v;
-  }
-  const float b = bias != nullptr ? bias[c] : 0.f;
-  constexpr int RB = 8;                    // rows whose loads are in flight together
-  for (int rb = 0; rb < nrows; rb += RB) {
-    float in[RB];
 #pragma unroll
-    for (int u = 0; u < RB; ++u)
-      in[u] = rb + u < nrows ? to_f(xc[(int64_t)(r0 + rb + u) * xs]) : 0.f;
+    for (int v = 0; v < VEC; ++v) win[j][v] = 0.f;
+    if (idx >= 0) load_channels<T, VEC>(xc + (int64_t)idx * xs, win[j]);
+    else if (!fresh) load_f32<VEC>(st + (int64_t)(K - 1 + idx) * C, win[j]);
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) old[j][v] = win[j][v];
+  }
+  constexpr int RB = VEC == 1 ? 8 : 4;     // rows whose loads are in flight together
+  for (int rb = 0; rb < nrows; rb += RB) {
+    float in[RB][VEC];
 #pragma unroll
     for (int u = 0; u < RB; ++u) {
-      const float cur = in[u];
-      float acc = b;
 #pragma unroll
-      for (int j = 0; j < K - 1; ++j) acc += wk[j] * win[j];
-      acc += wk[K - 1] * cur;
+      for (int v = 0; v < VEC; ++v) in[u][v] = 0.f;
+      if (rb + u < nrows) load_channels<T, VEC>(xc + (int64_t)(r0 + rb + u) * xs, in[u]);
+    }
 #pragma unroll
-      for (int j = 0; j + 1 < K - 1; ++j) win[j] = win[j + 1];
-      if constexpr (K > 1) win[K - 2] = cur;
-      if (rb + u < nrows) orow[(int64_t)(rb + u) * C] = silu ? acc * sigmoid_f(acc) : acc;
+    for (int u = 0; u < RB; ++u) {
+      float y[VEC];
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) {
+        float acc = b[v];
+#pragma unroll
+        for (int j = 0; j < K - 1; ++j) acc += wk[v][j] * win[j][v];
+        acc += wk[v][K - 1] * in[u][v];
+        y[v] = silu ? acc * sigmoid_f(acc) : acc;
+      }
+#pragma unroll
+      for (int j = 0; j + 1 < K - 1; ++j)
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) win[j][v] = win[j + 1][v];
+      if constexpr (K > 1) {
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) win[K - 2][v] = in[u][v];
+      }
+      if (rb + u < nrows) store_f32<VEC>(orow + (int64_t)(rb + u) * C, y);
     }
   }
   if (r0 == 0) {
@@ -130,16 +185,20 @@ __global__ __launch_bounds__(NT) void causal_conv_kernel(
 #pragma unroll
     for (int i = 0; i < K - 1; ++i) {
       const int idx = q.len - (K - 1) + i;
-      float v;
+      float v4[VEC];
       if (idx >= 0) {
-        v = to_f(xc[(int64_t)idx * xs]);
+        load_channels<T, VEC>(xc + (int64_t)idx * xs, v4);
       } else {
-        v = 0.f;
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) v4[v] = 0.f;
 #pragma unroll
         for (int j = 0; j < K - 1; ++j)
-          if (j == K - 1 + idx) v = old[j];
+          if (j == K - 1 + idx) {
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) v4[v] = old[j][v];
+          }
       }
-      st[(int64_t)i * C] = v;
+      store_f32<VEC>(st + (int64_t)i * C, v4);
     }
   }
 }
@@ -420,11 +479,21 @@ void launch_causal_conv(int dtype, float* out, const void* x, int64_t xs, const 
                         int C, int K, int num_slots, bool silu, hipStream_t s) {
   const int items = n_work * (blk_rows / CV_ROWS) + D;
   if (items <= 0 || C <= 0) return;
-  const dim3 grid(items, (C + NT - 1) / NT);
-#define KGC_CV(KK)                                                                           \
-  KGC_PM_DISPATCH_T(dtype, causal_conv_kernel<T, KK><<<grid, NT, 0, s>>>(                    \
+  // four channels per thread where every access is then an aligned 8- or 16-byte one
+  const int el = dtype == DT_F32 ? 4 : 2;
+  const bool vec = C % 4 == 0 && xs % 4 == 0 && reinterpret_cast<uintptr_t>(x) % (4 * el) == 0 &&
+                   reinterpret_cast<uintptr_t>(out) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(state) % 16 == 0;
+  const int per = NT * (vec ? 4 : 1);
+  const dim3 grid(items, (C + per - 1) / per);
+#define KGC_CV_V(KK, V)                                                                      \
+  KGC_PM_DISPATCH_T(dtype, causal_conv_kernel<T, KK, V><<<grid, NT, 0, s>>>(                 \
       out, (const T*)x, xs, w, bias, state, qsl, seq_lens, ctx_lens, slots, work_seq, work_blk, \
       n_work, blk_rows, P, Tp, C, num_slots, silu))
+#define KGC_CV(KK)                                    \
+  do {                                                \
+    if (vec) KGC_CV_V(KK, 4); else KGC_CV_V(KK, 1);   \
+  } while (0)
   switch (K) {
     case 1: KGC_CV(1); break;
     case 2: KGC_CV(2); break;
@@ -436,6 +505,7 @@ void launch_causal_conv(int dtype, float* out, const void* x, int64_t xs, const 
     default: KGC_CV(8); break;
   }
 #undef KGC_CV
+#undef KGC_CV_V
 }
 
 int matrix_scan_max_rows() { return 256; }

@@ -80,18 +80,21 @@ CUTS = [[200], [1], [2], [3, 1, 2, 70, 1, 1, 40, 2], [64, 65, 1], [17, 16, 15, 1
 # ---------------------------------------------------------------- convolution
 @pytest.mark.parametrize("dev", DEV)
 @pytest.mark.parametrize("K,bias", [(4, False), (3, True), (2, True), (5, False), (1, True)])
-def test_causal_conv_over_steps(dev, K, bias):
+@pytest.mark.parametrize("C,off,pad", [(37, 3, 5), (72, 8, 4)], ids=["odd", "aligned"])
+def test_causal_conv_over_steps(dev, K, bias, C, off, pad):
+    """Columns of a wider matrix at an odd offset, and at an offset, width and row stride
+    that are multiples of four (the GPU kernel then walks four channels per thread)."""
     dev = dev_of(dev)
     rng = np.random.default_rng(K)
-    n, C = 150, 37
+    n = 150
     x, w = rng.normal(size=(n, C)), rng.normal(size=(C, K))
     b = rng.normal(size=C) if bias else None
     want = oracle.silu(oracle.short_conv(x, w, b))
-    wide = f32(np.concatenate([rng.normal(size=(n, 3)), x, rng.normal(size=(n, 5))], 1), dev)
+    wide = f32(np.concatenate([rng.normal(size=(n, off)), x, rng.normal(size=(n, pad))], 1), dev)
     for cuts in CUTS:
         state = torch.full((4, max(K - 1, 1), C), 9.0, device=dev)    # another request's leftovers
         got = over_steps(n, cuts, dev, lambda lo, hi, m: ops.causal_conv(
-            wide[lo:hi, 3:3 + C], f32(w, dev), f32(b, dev) if bias else None, state, m))
+            wide[lo:hi, off:off + C], f32(w, dev), f32(b, dev) if bias else None, state, m))
         np.testing.assert_allclose(got, want, rtol=2e-5, atol=2e-5, err_msg=str(cuts))
         if K > 1:     # the state holds the last K - 1 inputs, oldest first
             np.testing.assert_allclose(state[2].cpu().numpy(), x[n - (K - 1):], rtol=1e-6, atol=1e-6)
