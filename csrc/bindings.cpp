@@ -1387,7 +1387,8 @@ void window_attention(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
                       std::optional<Tensor> dbt, std::optional<Tensor> work_seq,
                       std::optional<Tensor> work_blk, int64_t P, int64_t D, int64_t Tp,
                       double scale, int64_t window, int64_t keep_first,
-                      std::optional<Tensor> gate, bool fast, double softcap, double out_scale) {
+                      std::optional<Tensor> gate, bool fast, double softcap, double out_scale,
+                      std::optional<Tensor> elem_gate) {
   check_gpu(q, "q");
   c10::hip::HIPGuardMasqueradingAsCUDA g(q.device());
   TORCH_CHECK(q.dim() == 3 && q.is_contiguous() && act_dtype(q), "kgc.window_attention: q [T, H, dk]");
@@ -1421,7 +1422,18 @@ void window_attention(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
               out.size(1) == H * dv && out.stride(1) == 1 && (T <= 1 || out.stride(0) >= H * dv) &&
               out.scalar_type() == q.scalar_type(),
               "kgc.window_attention: out [T, H * dv] (rows may be slices of a wider buffer)");
-  const kgc::WindowExtra ex{T > 1 ? out.stride(0) : H * dv, (float)softcap, (float)out_scale};
+  const void* egp = nullptr;
+  int64_t egs = 0;
+  if (elem_gate.has_value()) {
+    TORCH_CHECK(elem_gate->is_cuda() && elem_gate->device() == q.device() && elem_gate->dim() == 2 &&
+                elem_gate->size(0) == T && elem_gate->size(1) == H * dv && elem_gate->stride(1) == 1 &&
+                elem_gate->scalar_type() == q.scalar_type(),
+                "kgc.window_attention: element-wise gate [T, H * dv] (a column slice)");
+    egp = elem_gate->data_ptr();
+    egs = elem_gate->stride(0);
+  }
+  const kgc::WindowExtra ex{T > 1 ? out.stride(0) : H * dv, (float)softcap, (float)out_scale, egp,
+                            egs};
   // the matrix-core kernel stores 8-byte pieces of a row
   const bool out_vec = reinterpret_cast<uintptr_t>(out.data_ptr()) % 8 == 0 &&
                        ex.ors * out.element_size() % 8 == 0;
@@ -1951,7 +1963,7 @@ TORCH_LIBRARY(kgc, m) {
   m.def("window_attention(Tensor(a!) out, Tensor q, Tensor k_cache, Tensor v_cache, Tensor? qsl, "
         "Tensor? seq_lens, Tensor? pbt, Tensor? ctx_lens, Tensor? dbt, Tensor? work_seq, Tensor? work_blk, "
         "int P, int D, int Tp, float scale, int window, int keep_first, Tensor? gate, bool fast, "
-        "float softcap, float out_scale) -> ()");
+        "float softcap, float out_scale, Tensor? elem_gate) -> ()");
   m.def("mlstm_scan(Tensor(a!) out, Tensor qkvg, Tensor gates, Tensor(b!) S, Tensor(c!) n, Tensor(d!) m, "
         "Tensor? qsl, Tensor? seq_lens, Tensor? ctx_lens, Tensor slots, int P, int D, int Tp, int H, int d, "
         "int dv) -> ()");

@@ -74,6 +74,14 @@ __device__ __forceinline__ float cap_score(float s, float cap) {
   return cap > 0.f ? cap * tanhf(s / cap) : s;
 }
 
+// sigmoid of the element-wise output gate at (row t, column c of the concatenated heads)
+template <typename T>
+__device__ __forceinline__ float elem_gate(const WindowExtra& ex, int64_t t, int c) {
+  if (ex.egate == nullptr) return 1.f;
+  const float g = to_f(static_cast<const T*>(ex.egate)[t * ex.egs + c]);
+  return 1.f / (1.f + expf(-g));
+}
+
 // grid (T, H), one wave.  LDS: q row [dk] fp32, p [64], value-row offsets [64].
 template <typename T>
 __global__ __launch_bounds__(64) void window_attention_kernel(
@@ -160,7 +168,7 @@ __global__ __launch_bounds__(64) void window_attention_kernel(
 #pragma unroll
   for (int u = 0; u < MAX_DV_PER_LANE; ++u) {
     const int c = lane + 64 * u;
-    if (c < dv) orow[c] = from_f<T>(acc[u] * inv);
+    if (c < dv) orow[c] = from_f<T>(acc[u] * inv * elem_gate<T>(ex, t, h * dv + c));
   }
 }
 
@@ -461,7 +469,8 @@ __global__ __launch_bounds__(64 * NWV) void window_decode_kernel(
       if (mw != -INFINITY) L += ml[w * QH + h] * expf(mw - M);
     }
     const float gt = (gate != nullptr ? gate[(int64_t)t * H + h0 + h] : 1.f) * ex.out_scale;
-    out[(int64_t)t * ex.ors + h0 * dv + e] = from_f<T>(accs[e] * gt / L);
+    out[(int64_t)t * ex.ors + h0 * dv + e] =
+        from_f<T>(accs[e] * gt / L * elem_gate<T>(ex, t, h0 * dv + e));
   }
 }
 
@@ -663,7 +672,9 @@ __global__ __launch_bounds__(256, KSM <= 4 ? 3 : 2) void window_prefill_mfma_ker
       if (t2 < ndt) {
         Pack4<T> w4;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) w4.h[i] = from_f<T>(o[t2][i] * inv);
+        for (int i = 0; i < 4; ++i)
+          w4.h[i] = from_f<T>(o[t2][i] * inv *
+                              elem_gate<T>(ex, q0 + myrow, h * dv + 16 * t2 + 4 * qd + i));
         *reinterpret_cast<u32x2*>(orow + 16 * t2 + 4 * qd) = w4.u;
       }
     }

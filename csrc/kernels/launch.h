@@ -271,11 +271,14 @@ void launch_rope_kv_store(int dtype, const void* qkv, int64_t qkv_stride,
 int window_attention_max_dv();
 // what an attention inside a wider mixer adds: the row stride of `out` in elements (its
 // rows may be column slices of a wider buffer), a tanh cap on the scaled scores (<= 0:
-// none), a factor on the result
+// none), a factor on the result, and an element-wise gate: the result is multiplied by
+// sigmoid(egate[t, head * dv + c]) (activation dtype, row stride egs; null: none)
 struct WindowExtra {
   int64_t ors;
   float softcap;
   float out_scale;
+  const void* egate;
+  int64_t egs;
 };
 void launch_window_attention(int dtype, void* out, const void* q, const void* k_cache,
                              const void* v_cache, const int* qsl, const int* seq_lens,

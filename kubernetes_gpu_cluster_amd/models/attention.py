@@ -200,8 +200,8 @@ class AttentionCore(nn.Module):
     v in the paged cache chosen at call time, attends causally (``spec.window`` when set)
     with scores q.k * scale that pass cap * tanh(. / cap) when ``spec.softcap`` > 0,
     multiplies the concatenated heads by sigmoid of the gate columns (``spec.elem_gate``)
-    and by ``out_scale``, and writes them into a column slice of the output projection's
-    input.  Softmax, scores and rotation are fp32."""
+    and by ``out_scale`` -- both in the attention kernels' epilogue -- and writes them into a
+    column slice of the output projection's input.  Softmax, scores and rotation are fp32."""
 
     def __init__(self, spec, out_scale: float = 1.0):
         super().__init__()
@@ -233,12 +233,7 @@ class AttentionCore(nn.Module):
                               sp.heads, sp.kv_heads, sp.dim, sp.vdim,
                               bool(sp.rotary and sp.rotary.interleaved))
         w = sp.window
-        if not sp.elem_gate:
-            ops.window_attention(q, kc, vc, positions, ctx.attn, self.scale,
-                                 w.size if w else 0, w.keep_first if w else 0, None,
-                                 sp.softcap, self.out_scale, out=out)
-            return
-        o = ops.window_attention(q, kc, vc, positions, ctx.attn, self.scale,
-                                 w.size if w else 0, w.keep_first if w else 0, None, sp.softcap)
-        g = proj[:, col0 + self.n_qkv: col0 + self.n_in]
-        ops.gate_mul(o.view(o.shape[0], sp.heads, sp.vdim), g, self.out_scale, out=out)
+        g = proj[:, col0 + self.n_qkv: col0 + self.n_in] if sp.elem_gate else None
+        ops.window_attention(q, kc, vc, positions, ctx.attn, self.scale, w.size if w else 0,
+                             w.keep_first if w else 0, None, sp.softcap, self.out_scale, out=out,
+                             elem_gate=g)

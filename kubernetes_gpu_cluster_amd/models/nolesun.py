@@ -20,7 +20,7 @@ fp32.
 
 Kernel sequence per layer run (ops/__init__.py, "parallel mixers"):
   residual_norm (the previous sublayer's normed result joins x; norm) -> ONE merged
-  projection GEMM for both mixers -> rope_kv_store -> window_attention (-> gate_mul) |
+  projection GEMM for both mixers -> rope_kv_store -> window_attention (gate in its epilogue) |
   causal_conv -> ssd_scan / gated_delta_scan -> gated_rms_norm, both writing column slices
   of one buffer -> ONE output GEMM over [left | right] (the mixers' scales ride on the
   activations) -> residual_norm -> feed-forward (up GEMM -> relu_sq -> down GEMM | gate_proj

@@ -714,12 +714,14 @@ def window_attention_fast() -> bool:
 def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                      positions: torch.Tensor, meta, scale: float, window: int, keep_first: int,
                      gate: Optional[torch.Tensor] = None, softcap: float = 0.0,
-                     out_scale: float = 1.0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                     out_scale: float = 1.0, out: Optional[torch.Tensor] = None,
+                     elem_gate: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Prefill chunks and decode rows of one step alike: row t sees the cached keys
     j <= p with p - j < window or j < keep_first (p = positions[t]; window <= 0: plain
     causal).  Decode padding rows (context length 0) give zeros.  ``softcap`` > 0: the
     scaled scores pass softcap * tanh(. / softcap).  The result is multiplied by
-    ``out_scale`` and may go to ``out`` [T, H * dv], a column slice of a wider buffer."""
+    sigmoid(``elem_gate`` [T, H * dv], a column slice of a projection) when given and by
+    ``out_scale``, and may go to ``out`` [T, H * dv], a column slice of a wider buffer."""
     T, H, _ = q.shape
     dv = v_cache.shape[3]
     if not _gpu(q):
@@ -728,7 +730,7 @@ def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
             tp = meta.num_prefill_tokens
             pos[tp:tp + meta.num_decodes] = meta.decode_ctx_lens[: meta.num_decodes].long() - 1
         r = ref.window_attention(q, k_cache, v_cache, pos, _row_tables(meta, T), scale,
-                                 window, keep_first, gate, softcap, out_scale)
+                                 window, keep_first, gate, softcap, out_scale, elem_gate)
         if out is not None:
             out.copy_(r)
             return out
@@ -747,7 +749,7 @@ def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
                           meta.decode_ctx_lens, meta.decode_block_tables, ws, wb,
                           meta.num_prefills, meta.num_decodes, meta.num_prefill_tokens,
                           scale, window, keep_first, gate, window_attention_fast(),
-                          float(softcap), float(out_scale))
+                          float(softcap), float(out_scale), elem_gate)
     return out
 
 

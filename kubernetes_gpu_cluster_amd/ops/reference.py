@@ -455,13 +455,15 @@ def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
                      positions: torch.Tensor, row_tables: torch.Tensor, scale: float,
                      window: int, keep_first: int,
                      gate: Optional[torch.Tensor], softcap: float = 0.0,
-                     out_scale: float = 1.0) -> torch.Tensor:
+                     out_scale: float = 1.0,
+                     elem_gate: Optional[torch.Tensor] = None) -> torch.Tensor:
     """q [T, H, dk] (rotated; the step's k / v already stored) -> [T, H*dv].  Row t at
     position p = positions[t] attends the cached keys j <= p with p - j < window or
     j < keep_first (window <= 0: all of them) of the sequence whose block table is
     row_tables[t]; scores q.k * scale, then softcap * tanh(score / softcap) when
     softcap > 0; softmax and the weighted sum in fp32; each head's output times
-    gate[t, head] (fp32) when given, and times out_scale."""
+    gate[t, head] (fp32) when given, the concatenated heads times sigmoid(elem_gate
+    [T, H*dv]) when given, and times out_scale."""
     T, H, dk = q.shape
     G, bs, dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[3]
     out = torch.zeros(T, H, dv, dtype=torch.float32)
@@ -483,6 +485,8 @@ def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
         out[t] = torch.einsum("ghn,ngv->ghv", pr, v).reshape(H, dv)
     if gate is not None:
         out = out * gate.float()[:, :, None]
+    if elem_gate is not None:
+        out = out * torch.sigmoid(elem_gate.float()).view(T, H, dv)
     if out_scale != 1.0:
         out = out * out_scale
     return out.view(T, H * dv).to(q.dtype)
