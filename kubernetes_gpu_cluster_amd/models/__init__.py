@@ -20,6 +20,7 @@ from .configs import PRESETS, ModelConfig, resolve_model
 from .dilavik import DilavikForCausalLM
 from .konovik import KonovikForCausalLM
 from .llama import LlamaForCausalLM
+from .lorenex import LorenexForCausalLM
 from .nolesun import NolesunForCausalLM
 from .opt import OPTForCausalLM
 
@@ -33,6 +34,8 @@ def build_model(cfg: ModelConfig, dtype=torch.bfloat16, device=None):
         return KonovikForCausalLM(cfg, dtype, device)
     if cfg.arch == "nolesun":
         return NolesunForCausalLM(cfg, dtype, device)
+    if cfg.arch == "lorenex":
+        return LorenexForCausalLM(cfg, dtype, device)
     return LlamaForCausalLM(cfg, dtype, device)
 
 

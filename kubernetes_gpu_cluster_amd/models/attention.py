@@ -201,11 +201,17 @@ class AttentionCore(nn.Module):
     with scores q.k * scale that pass cap * tanh(. / cap) when ``spec.softcap`` > 0,
     multiplies the concatenated heads by sigmoid of the gate columns (``spec.elem_gate``)
     and by ``out_scale`` -- both in the attention kernels' epilogue -- and writes them into a
-    column slice of the output projection's input.  Softmax, scores and rotation are fp32."""
+    column slice of the output projection's input.  Softmax, scores and rotation are fp32.
 
-    def __init__(self, spec, out_scale: float = 1.0):
+    With ``spec.conv`` taps, q | k | v first pass a causal convolution over time per channel
+    (no bias, no activation; the last taps - 1 projected rows are per-sequence state).
+    ``spec.qk_unit`` / ``spec.v_unit`` divide each head's q and k / v by its root mean square
+    (v is cached so), and ``spec.q_temp`` = (coef, every) multiplies q at position p by
+    1 + coef * ln(floor((p + 1) / every) + 1); these take the place of the rotation."""
+
+    def __init__(self, spec, out_scale: float = 1.0, eps: float = 1e-6, device=None):
         super().__init__()
-        self.spec, self.out_scale = spec, float(out_scale)
+        self.spec, self.out_scale, self.eps = spec, float(out_scale), eps
         H, G, dk, dv = spec.heads, spec.kv_heads, spec.dim, spec.vdim
         assert H % G == 0, "query heads must be a multiple of key/value heads"
         assert spec.rot_dims % 2 == 0 and spec.rot_dims <= dk
@@ -214,6 +220,16 @@ class AttentionCore(nn.Module):
         self.n_out = H * dv
         self.scale = spec.dim ** -0.5 if spec.scale is None else spec.scale
         self.rope = None            # [max_pos, rot_dims] fp32, set by prepare()
+        self.unit = bool(spec.qk_unit or spec.v_unit or spec.q_temp)
+        assert not (self.unit and spec.rot_dims), "unit-RMS inputs take the rotation's place"
+        self.conv_w = (nn.Parameter(torch.zeros(self.n_qkv, spec.conv, dtype=torch.float32,
+                                                device=device), requires_grad=False)
+                       if spec.conv else None)
+
+    def state_shapes(self) -> tuple:
+        """Per-slot shapes of the state tensors: the convolution's last inputs, if any."""
+        sp = self.spec
+        return ((max(sp.conv - 1, 1), self.n_qkv),) if sp.conv else ()
 
     def prepare(self, tables: dict, max_pos: int, device) -> None:
         sp = self.spec
@@ -225,13 +241,21 @@ class AttentionCore(nn.Module):
         self.rope = tables[key]
 
     def forward(self, proj: torch.Tensor, col0: int, positions: torch.Tensor,
-                ctx: ForwardContext, cache_idx: int, out: torch.Tensor) -> None:
+                ctx: ForwardContext, cache_idx: int, out: torch.Tensor,
+                state: tuple = ()) -> None:
         sp = self.spec
         kc, vc = ctx.kv_caches[cache_idx]
         qkv = proj[:, col0: col0 + self.n_qkv]
-        q = ops.rope_kv_store(qkv, positions, self.rope, kc, vc, ctx.attn.slot_mapping,
-                              sp.heads, sp.kv_heads, sp.dim, sp.vdim,
-                              bool(sp.rotary and sp.rotary.interleaved))
+        if self.conv_w is not None:
+            qkv = ops.causal_conv(qkv, self.conv_w, None, state[0], ctx.attn, False)
+        if self.unit:
+            q = ops.norm_kv_store(qkv.float(), positions, kc, vc, ctx.attn.slot_mapping, sp.heads,
+                                  sp.kv_heads, sp.dim, sp.vdim, self.eps, sp.qk_unit, sp.v_unit,
+                                  sp.q_temp, proj.dtype)
+        else:
+            q = ops.rope_kv_store(qkv.to(proj.dtype), positions, self.rope, kc, vc,
+                                  ctx.attn.slot_mapping, sp.heads, sp.kv_heads, sp.dim, sp.vdim,
+                                  bool(sp.rotary and sp.rotary.interleaved))
         w = sp.window
         g = proj[:, col0 + self.n_qkv: col0 + self.n_in] if sp.elem_gate else None
         ops.window_attention(q, kc, vc, positions, ctx.attn, self.scale, w.size if w else 0,

@@ -58,8 +58,17 @@ class FeedForwardSpec:
     # form (dense: gated, moe: ungated)
     gated: Optional[bool] = None
     # "sigmoid": the routing described above; "softmax": logits W_r h + b_r, the ``top``
-    # largest chosen, their weights the softmax over the chosen logits only
+    # largest chosen, their weights the softmax over the chosen logits only; "softmax_all":
+    # scores = softmax over all router outputs, the choice made on score + a per-output
+    # correction, the weights the chosen scores as they are
     router: str = "sigmoid"
+    # act "polynorm" (dense, not gated): a N(z) + b N(z^2) + c N(z^3) + e with N = division
+    # by the row's root mean square and four learned numbers.  act "swiglu_clamp" (gated):
+    # g = min(gate h, limit), u = clamp(up h, -limit, limit), g sigmoid(1.702 g) (u + 1)
+    limit: float = 0.0
+    # the last ``identity`` router outputs (beyond ``experts``) name experts without weights
+    # whose output is their input
+    identity: int = 0
 
 
 @dataclasses.dataclass(frozen=True)
@@ -86,7 +95,14 @@ class MixerSpec:
     x | B | C, a SiLU gate before an RMS norm in ``inner_norm_groups`` parts.
     kind "gated_delta": the gated delta rule, ``heads`` value heads over ``kv_heads``
     query / key heads, a [dim, vdim] fp32 state per head, convolutions of ``conv`` taps
-    without bias on q, k and v, a per-head RMS norm and a SiLU gate after it."""
+    without bias on q, k and v, a per-head RMS norm and a SiLU gate after it.
+    kind "gla": gated linear attention, per head S = diag(alpha) S + k v^T, o = S^T q with a
+    decay per key channel alpha = sigmoid(W_a2 W_a1 h + b)^(1 / decay_tau) through a
+    bottleneck of ``decay_rank``; a per-head RMS norm and a SiLU gate after it.
+    kind "mamba": the selective scan, ``width`` channels with ``dim`` states each
+    (S[c, n] = exp(dt_c A[c, n]) S[c, n] + dt_c x_c B_n, y_c = S[c, :] . C + D_c x_c), step
+    sizes through a bottleneck of ``dt_rank``, a causal convolution of ``conv`` taps with
+    bias and SiLU on x, a SiLU gate on the result."""
     kind: str
     heads: int
     dim: int
@@ -112,6 +128,18 @@ class MixerSpec:
     elem_gate: bool = False
     conv: int = 0                # mamba2 / gated_delta: taps of the causal convolution
     inner_norm_groups: int = 1   # mamba2: parts of the gated RMS norm
+    # attention inside a parallel mixer: a causal convolution of ``conv`` taps (no bias, no
+    # activation) on q, k and v right after the projection; q and k (``qk_unit``) and v
+    # (``v_unit``) divided by their root mean square per head; q times
+    # 1 + coef * ln(floor((p + 1) / every) + 1) at position p (``q_temp`` = (coef, every));
+    # ``out_bias``: whether the output projection has a bias (None: as ``bias``)
+    qk_unit: bool = False
+    v_unit: bool = False
+    q_temp: Optional[tuple] = None
+    out_bias: Optional[bool] = None
+    decay_tau: float = 1.0       # gla
+    decay_rank: int = 0
+    dt_rank: int = 0             # mamba
     left: Optional["MixerSpec"] = None      # parallel
     right: Optional["MixerSpec"] = None
     left_scale: float = 1.0
@@ -170,6 +198,10 @@ class ModelConfig:
     # it joins the stream (norm weights stored around zero); before each pass of the loop
     # x <- W_in [x; embedding output] + step[pass]
     loop_mix: bool = False
+    # arch "lorenex": sublayers read the stream itself and their RMS-normed results join it
+    # times ``residual_mult``; a learned position vector is added to the scaled embedding;
+    # layer i runs with the weights of layer ``weights_of[i]`` (cache and state its own)
+    weights_of: Optional[tuple] = None
 
     @property
     def q_size(self) -> int:
@@ -204,7 +236,9 @@ class ModelConfig:
         h, i, L = self.hidden_size, self.intermediate_size, self.num_layers
         if self.layer_specs:
             n = 2 * self.vocab_size * h
-            for sp in self.layer_specs:
+            for li, sp in enumerate(self.layer_specs):
+                if self.weights_of and self.weights_of[li] != li:
+                    continue                # a layer that runs with another layer's tensors
                 if sp.kind == "latent_attention":
                     n += h * (sp.heads * (sp.dim + sp.rot_dims) + sp.kv_rank + sp.rot_dims)
                     n += sp.kv_rank * sp.heads * (sp.dim + sp.vdim) + 2 * h * sp.heads * sp.vdim
@@ -216,10 +250,15 @@ class ModelConfig:
                     n += l.heads * l.vdim * h * (2 if l.elem_gate else 1)
                     if r.kind == "mamba2":
                         n += h * (3 * r.heads * r.vdim + 2 * r.kv_heads * r.dim + r.heads)
+                    elif r.kind == "mamba":
+                        n += 3 * h * r.width + r.width * (2 * r.dt_rank + 3 * r.dim)
                     else:
                         n += h * (2 * r.kv_heads * r.dim + 3 * r.heads * r.vdim + 2 * r.heads)
                 elif sp.kind == "attention":
                     n += h * (sp.heads * sp.dim + sp.kv_heads * (sp.dim + sp.vdim) + sp.heads)
+                elif sp.kind == "gla":
+                    n += h * (2 * sp.heads * sp.dim + 3 * sp.heads * sp.vdim)
+                    n += sp.decay_rank * (h + sp.heads * sp.dim)
                 else:
                     n += h * (2 * sp.heads * sp.dim + 2 * sp.heads * sp.vdim + 2 * sp.heads)
                 if sp.kind in ("attention", "mlstm"):
@@ -231,7 +270,7 @@ class ModelConfig:
                     n += (2 if f.gated is False else 3) * h * f.ff
                 else:
                     n += ((3 if f.gated else 2) * h * f.experts * f.ff + 2 * h * f.shared_ff
-                          + h * (f.experts + 1))
+                          + h * (f.experts + f.identity + 1))
                 n += 2 * h * self.side_dim
             return n + self.vocab_size * self.side_dim * len(self.layer_specs)
         attn = h * (self.q_size + 2 * self.kv_size) + self.q_size * h
@@ -457,6 +496,64 @@ PRESETS.update({
 })
 
 
+def _lorenex(name: str, width: int, pattern: str, gla: dict, att: dict, ssm: dict, dense_ff: int,
+             expert_ff: int, experts: int = 8, top: int = 2, identity: int = 1,
+             vocab: int = 32000, share: Optional[dict] = None, max_pos: int = 8192) -> ModelConfig:
+    """A Lorenex-architecture preset: ``pattern`` is one letter per layer ("g": gated linear
+    attention, "p": attention beside the selective scan; a capital letter: routed experts
+    instead of the dense feed-forward); ``share`` maps a layer to the layer whose weights
+    it runs with."""
+    dense = FeedForwardSpec("dense", dense_ff, act="polynorm", gated=False)
+    moe = FeedForwardSpec("moe", expert_ff, act="swiglu_clamp", gated=True, experts=experts,
+                          top=top, router="softmax_all", limit=7.0, identity=identity)
+    specs = []
+    for c in pattern:
+        mlp = moe if c.isupper() else dense
+        if c.lower() == "g":
+            specs.append(MixerSpec("gla", gla["heads"], gla["dim"], gla["vdim"], ff=mlp.ff, mlp=mlp,
+                                   decay_tau=gla.get("tau", 16.0), decay_rank=gla.get("rank", 16)))
+            continue
+        left = MixerSpec("attention", att["heads"], att["dim"], att["vdim"], kv_heads=att["kv"],
+                         scale=att.get("scale", 1.0), bias=True, out_bias=False,
+                         conv=att.get("conv", 4), qk_unit=True, v_unit=True,
+                         q_temp=(att.get("coef", 0.5), att.get("every", 1024)))
+        right = MixerSpec("mamba", 1, ssm["state"], ssm["inner"], width=ssm["inner"],
+                          conv=ssm.get("conv", 4), dt_rank=ssm["dt_rank"])
+        specs.append(MixerSpec("parallel", left.heads, left.dim, left.vdim, kv_heads=left.kv_heads,
+                               ff=mlp.ff, mlp=mlp, left=left, right=right, left_scale=1.0,
+                               right_scale=1.0))
+    share = share or {}
+    return ModelConfig(name, "lorenex", len(specs), width, att["heads"], att["kv"], att["dim"],
+                       dense_ff, vocab, max_position=max_pos, rms_eps=1e-5, tie_embeddings=True,
+                       learned_pos=True, layer_specs=tuple(specs), embed_scale=width ** 0.5,
+                       residual_mult=0.5,
+                       weights_of=tuple(share.get(i, i) for i in range(len(specs))),
+                       bos_token_id=1, eos_token_id=2)
+
+
+# Lorenex presets beside the equal-width hybrid / Llama presets above: the same number of
+# layers, 16 / 32 attention heads of 128, a feed-forward whose active parameters per token are
+# those of the Llama preset's (the two-matrix dense one 1.5 x as wide as the gated one; two of
+# eight gated experts of half its size, plus an identity expert).  Gated-linear-attention
+# layers have key size width / 2 and value size width; the selective scan beside the
+# attention is as wide as the model with 16 states per channel.
+PRESETS.update({
+    "lorenex-w2048": _lorenex("lorenex-w2048", 2048, "gPgPgPgPgPgP",
+                              dict(heads=8, dim=128, vdim=256, rank=16),
+                              dict(heads=16, kv=4, dim=128, vdim=128, scale=12.0),
+                              dict(inner=2048, state=16, dt_rank=128), 8256, 2752),
+    "lorenex-w4096": _lorenex("lorenex-w4096", 4096, "gPgPgPgP",
+                              dict(heads=16, dim=128, vdim=256, rank=16),
+                              dict(heads=32, kv=8, dim=128, vdim=128, scale=12.0),
+                              dict(inner=4096, state=16, dt_rank=256), 21504, 7168),
+    "tiny-lorenex": _lorenex("tiny-lorenex", 128, "gPpG",
+                             dict(heads=2, dim=16, vdim=32, rank=4, tau=8.0),
+                             dict(heads=4, kv=2, dim=32, vdim=16, scale=6.0, conv=3, every=16),
+                             dict(inner=96, state=8, dt_rank=6, conv=3), 192, 64, experts=4,
+                             vocab=1024, share={2: 1}, max_pos=2048),
+})
+
+
 # HF repo basenames (lower-cased) -> preset
 _ALIASES = {
     "meta-llama-3-8b": "llama-3-8b", "meta-llama-3-8b-instruct": "llama-3-8b",
@@ -631,8 +728,95 @@ def nolesun_config(d: dict, name: str) -> ModelConfig:
         bos_token_id=int(d.get("bos_token_id", 0)), eos_token_id=int(d.get("eos_token_id", -1)))
 
 
-def _from_hf_config(d: dict, name: str) -> ModelConfig:
+def _lorenex_ff(mlp: Optional[dict]) -> Optional[FeedForwardSpec]:
+    if not mlp:
+        return None
+    kind = mlp.get("kind", "dense")
+    if kind == "dense":
+        return FeedForwardSpec("dense", int(mlp["ff"]), act="polynorm", gated=False)
+    if kind == "moe":
+        rt, ex = mlp["router"], mlp["expert"]
+        return FeedForwardSpec("moe", int(ex["ff"]), act="swiglu_clamp", gated=True,
+                               experts=int(rt["experts"]), top=int(rt["top"]),
+                               router="softmax_all", limit=float(ex["limit"]),
+                               identity=int(rt.get("identity", 0)))
+    raise ValueError(f"unsupported feed-forward kind {kind!r}")
+
+
+def _lorenex_spec(entry: dict, rank: Optional[int]) -> MixerSpec:
+    """One entry of a Lorenex ``layers`` list.  ``rank``: the bottleneck of a gated-linear-
+    attention layer's decay projection, which only its tensors' shapes give."""
+    kind, m = entry["type"], entry["mixer"]
+    mlp = _lorenex_ff(entry.get("mlp"))
+    ff = mlp.ff if mlp else 0
+    if kind == "gla":
+        rank = int(m["rank"]) if "rank" in m else rank
+        if not rank:
+            raise ValueError("a gla layer needs its decay bottleneck: mixer.rank in the config, "
+                             "or the checkpoint whose <layer>.mix.a1 has that many rows")
+        return MixerSpec("gla", int(m["heads"]), int(m["dim"]), int(m["vdim"]), ff=ff, mlp=mlp,
+                         decay_tau=float(m["tau"]), decay_rank=rank)
+    if kind != "parallel":
+        raise ValueError(f"unknown mixer type {kind!r}")
+    l, r = m["left"], m["right"]
+    qt = l.get("q_temp")
+    H = int(l["heads"])
+    left = MixerSpec("attention", H, int(l["dim"]), int(l["vdim"]),
+                     kv_heads=int(l.get("kv_heads", H)), scale=float(l["scale"]), bias=True,
+                     out_bias=False, conv=int(l.get("conv", 1)), qk_unit=True, v_unit=True,
+                     q_temp=(float(qt["coef"]), int(qt["every"])) if qt else None)
+    if left.heads % left.kv_heads:
+        raise ValueError("heads must be a multiple of the key/value heads")
+    right = MixerSpec("mamba", 1, int(r["state"]), int(r["inner"]), width=int(r["inner"]),
+                      conv=int(r["conv"]), dt_rank=int(r["dt_rank"]))
+    return MixerSpec("parallel", H, left.dim, left.vdim, kv_heads=left.kv_heads, ff=ff, mlp=mlp,
+                     left=left, right=right, left_scale=float(m.get("left_scale", 1.0)),
+                     right_scale=float(m.get("right_scale", 1.0)))
+
+
+def lorenex_config(d: dict, name: str, shapes: Optional[dict] = None) -> ModelConfig:
+    """A Lorenex config.json (``architecture``, ``width``, ``vocab``, ``max_positions``,
+    ``layers``, ``norm``, ``embedding``, ``residual_mult``) -> ModelConfig.  ``shapes``:
+    tensor name -> shape of the checkpoint beside it, for the sizes config.json leaves to
+    the tensors."""
+    layers = d["layers"]
+    share = tuple(int(e.get("weights_of", i)) for i, e in enumerate(layers))
+    for i, j in enumerate(share):
+        if not 0 <= j < len(layers) or share[j] != j or layers[j]["type"] != layers[i]["type"]:
+            raise ValueError(f"layer {i}: bad weights_of {j}")
+    specs = []
+    for i, e in enumerate(layers):
+        a1 = (shapes or {}).get(f"l{share[i]}.mix.a1")
+        specs.append(_lorenex_spec(e, int(a1[0]) if a1 else None))
+    a = next((sp.left for sp in specs if sp.kind == "parallel"), specs[0])
+    return ModelConfig(
+        name, "lorenex", len(specs), int(d["width"]), a.heads, a.kv_heads or a.heads, a.dim,
+        max((sp.ff for sp in specs), default=0), int(d["vocab"]),
+        max_position=int(d.get("max_positions", 8192)), rms_eps=float(d["norm"]["eps"]),
+        tie_embeddings=True, learned_pos=True, layer_specs=tuple(specs),
+        embed_scale=float(d.get("embedding", {}).get("scale", 1.0)),
+        residual_mult=float(d.get("residual_mult", 1.0)), weights_of=share,
+        bos_token_id=int(d.get("bos_token_id", 0)), eos_token_id=int(d.get("eos_token_id", -1)))
+
+
+def _tensor_shapes(path: str) -> dict:
+    """Tensor name -> shape from the headers of the safetensors files in ``path``."""
+    import glob
+    import struct
+    shapes = {}
+    for fn in sorted(glob.glob(os.path.join(path, "*.safetensors"))):
+        with open(fn, "rb") as f:
+            (n,) = struct.unpack("<Q", f.read(8))
+            for k, v in json.loads(f.read(n)).items():
+                if k != "__metadata__":
+                    shapes[k] = tuple(v["shape"])
+    return shapes
+
+
+def _from_hf_config(d: dict, name: str, path: Optional[str] = None) -> ModelConfig:
     """Map an HF config.json dict onto ModelConfig."""
+    if d.get("architecture") == "Lorenex":
+        return lorenex_config(d, name, _tensor_shapes(path) if path else None)
     if d.get("architecture") == "Nolesun":
         return nolesun_config(d, name)
     if d.get("architecture") == "Dilavik":
@@ -683,7 +867,7 @@ def resolve_model(model: str) -> tuple[ModelConfig, Optional[str]]:
         return PRESETS[key], None
     if os.path.isdir(model) and os.path.isfile(os.path.join(model, "config.json")):
         with open(os.path.join(model, "config.json")) as f:
-            cfg = _from_hf_config(json.load(f), os.path.basename(model.rstrip("/")))
+            cfg = _from_hf_config(json.load(f), os.path.basename(model.rstrip("/")), model)
         return cfg, model
     base = os.path.basename(key)
     base = _ALIASES.get(base, base)

@@ -359,3 +359,56 @@ class SoftmaxRoutedExperts(nn.Module):
         a = ops.silu_mul(torch.bmm(xe, self.w13.transpose(1, 2)))
         dense = torch.bmm(a, self.w2.transpose(1, 2))
         return ops.moe_finish(None, dense, topk_w, topk_ids, None, None)
+
+
+class SoftmaxAllRoutedExperts(nn.Module):
+    """Mixture of clamped gated experts with softmax routing over all router outputs:
+    scores s = softmax(W_r h) in fp32 over ``experts + identity`` outputs; the ``top`` with
+    the largest s + correction are chosen and weighted by s as it is (no renormalisation).
+    An expert is down(g sigmoid(1.702 g) (u + 1)) with g = min(gate h, limit) and
+    u = clamp(up h, -limit, limit); the last ``identity`` router outputs name experts without
+    weights whose output is the token's input itself.  Expert weights are kept as
+    w13 [E, 2 ff, hidden] (gate rows, then up rows) and w2 [E, hidden, ff].
+
+    Expert GEMMs: the grouped MFMA GEMM over expert-sorted rows where its tiles cover the
+    shapes (16-bit activations, 2 ff % 128 == 0, hidden % 128 == 0, ff % 64 == 0; pairs of
+    identity experts fall outside the expert range and add nothing there); otherwise every
+    expert runs on every token as one batched GEMM pair and the chosen outputs are gathered.
+    The identity experts' share, (sum of their chosen scores) * h, joins in the finishing
+    kernel.  No host synchronisation, so decode graphs capture the block.  One GPU per
+    replica."""
+
+    def __init__(self, hidden: int, spec, dtype, device):
+        super().__init__()
+        assert spec.act == "swiglu_clamp" and spec.gated and spec.router == "softmax_all"
+        self.spec = spec
+        E, I = spec.experts, spec.ff
+        z = lambda *s: nn.Parameter(torch.zeros(*s, dtype=dtype, device=device),   # noqa: E731
+                                    requires_grad=False)
+        self.w13 = z(E, 2 * I, hidden)
+        self.w2 = z(E, hidden, I)
+        self.router = z(E + spec.identity, hidden)
+        self.correction = nn.Parameter(torch.zeros(E + spec.identity, dtype=torch.float32,
+                                                   device=device), requires_grad=False)
+        self.native = (torch.device(device).type == "cuda" and dtype != torch.float32 and
+                       ops.moe_supported(2 * I, hidden) and ops.moe_supported(hidden, I))
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        sp = self.spec
+        logits = ops.gate_proj(x, self.router, None, ops.GATE_NONE)        # fp32 [T, E + identity]
+        topk_w, topk_ids, idw = ops.moe_route_softmax_all(logits, self.correction, sp.top,
+                                                          sp.experts)
+        act = lambda t: ops.swiglu_clamp(t, sp.limit)                      # noqa: E731
+        routed = dense = None
+        if self.native and x.is_cuda:
+            routed = ops.grouped_experts(x, self.w13, self.w2, topk_w, topk_ids, act,
+                                         all_local=sp.identity == 0)
+            if not sp.identity:
+                return routed
+        else:
+            T = x.shape[0]
+            xe = x.unsqueeze(0).expand(sp.experts, T, x.shape[1])
+            dense = torch.bmm(act(torch.bmm(xe, self.w13.transpose(1, 2))), self.w2.transpose(1, 2))
+        if sp.identity:
+            return ops.moe_finish(routed, dense, topk_w, topk_ids, x, idw)
+        return ops.moe_finish(None, dense, topk_w, topk_ids, None, None)

@@ -41,7 +41,7 @@ from ..parallel.state import get_state
 from .attention import AttentionCore, ForwardContext
 from .configs import ModelConfig
 from .moe import SoftmaxRoutedExperts
-from .recurrent import GatedDeltaCore, Mamba2Core
+from .recurrent import GatedDeltaCore, Mamba2Core, MambaCore
 
 
 def _f32(shape, device, fill=0.0):
@@ -66,37 +66,46 @@ class ParallelMixer(nn.Module):
     left_scale * left(h) + right_scale * right(h).  Both mixers' input projections are one
     GEMM (left columns first), and both output projections one GEMM over the concatenated
     [left | right] features; the scales are applied to those features in fp32 before they
-    are rounded, so the weights stay the checkpoint's."""
+    are rounded, so the weights stay the checkpoint's.  The right mixer is Mamba-2, the gated
+    delta rule or the selective scan; a layer run's state tensors are the left mixer's (its
+    convolution inputs, if it has any) followed by the right mixer's."""
 
     def __init__(self, hidden: int, spec, eps: float, dtype, device):
         super().__init__()
         self.spec = spec
         l, r = spec.left, spec.right
-        self.left = AttentionCore(l, spec.left_scale)
-        core = Mamba2Core if r.kind == "mamba2" else GatedDeltaCore
-        self.right = core(r, eps, device, spec.right_scale)
+        self.left = AttentionCore(l, spec.left_scale, eps, device)
+        if r.kind == "mamba":
+            self.right = MambaCore(r, eps, device, spec.right_scale, dtype)
+        else:
+            core = Mamba2Core if r.kind == "mamba2" else GatedDeltaCore
+            self.right = core(r, eps, device, spec.right_scale)
+        o_bias = l.bias if l.out_bias is None else l.out_bias
         self.in_proj = ReplicatedLinear(hidden, self.left.n_in + self.right.n_in, bias=l.bias,
                                         dtype=dtype, device=device)
-        self.o_proj = ReplicatedLinear(self.left.n_out + self.right.n_out, hidden, bias=l.bias,
+        self.o_proj = ReplicatedLinear(self.left.n_out + self.right.n_out, hidden, bias=o_bias,
                                        dtype=dtype, device=device)
         if l.bias:                  # only the left mixer's columns carry a bias
             self.in_proj.bias.data.zero_()
+        if o_bias:
             self.o_proj.bias.data.zero_()
+        self.n_left_state = len(self.left.state_shapes())
 
     def cache_shape(self) -> tuple:
         l = self.spec.left
         return (l.kv_heads, l.dim, l.vdim)
 
     def state_shapes(self) -> tuple:
-        return self.right.state_shapes()
+        return self.left.state_shapes() + self.right.state_shapes()
 
     def forward(self, h: torch.Tensor, positions: torch.Tensor, ctx: ForwardContext,
                 cache_idx: int, state: tuple) -> torch.Tensor:
         proj = self.in_proj(h)
         feats = torch.empty(h.shape[0], self.left.n_out + self.right.n_out, dtype=h.dtype,
                             device=h.device)
-        self.left(proj, 0, positions, ctx, cache_idx, feats[:, : self.left.n_out])
-        self.right(proj, self.left.n_in, ctx, state, feats[:, self.left.n_out:])
+        nl = self.n_left_state
+        self.left(proj, 0, positions, ctx, cache_idx, feats[:, : self.left.n_out], state[:nl])
+        self.right(proj, self.left.n_in, ctx, state[nl:], feats[:, self.left.n_out:])
         return self.o_proj(feats)
 
 

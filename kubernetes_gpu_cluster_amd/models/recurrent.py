@@ -166,3 +166,86 @@ class GatedDeltaCore(nn.Module):
         o = ops.gated_delta_scan(qkv, ba, self.a_log, self.dt_bias, state[1], ctx.attn,
                                  sp.heads, sp.kv_heads, sp.dim, sp.vdim)
         ops.gated_rms_norm(o, g, self.norm_weight, sp.heads, self.eps, False, out)
+
+
+class GLAMixer(nn.Module):
+    """Gated linear attention: per head a [dim, vdim] fp32 state with one decay per key
+    channel.  q = W_q h * dim^-1/2, k = W_k h, v = W_v h;
+    alpha = sigmoid(W_a2 (W_a1 h) + b)^(1 / tau), laid out heads x dim;
+        S = diag(alpha) S + k v^T,   o = S^T q
+    then each head's o over its RMS, times a weight shared by the heads, the concatenated
+    heads times silu(W_g h), and the output projection.  One merged projection yields
+    q | k | v | g | the decay bottleneck; the second decay projection (a few columns wide)
+    runs inside the scan kernel in fp32, so the decay's logarithm never passes 16 bits."""
+
+    def __init__(self, hidden: int, spec, eps: float, dtype, device):
+        super().__init__()
+        self.spec, self.eps = spec, eps
+        H, d, dv, r = spec.heads, spec.dim, spec.vdim, spec.decay_rank
+        assert r >= 1
+        self.n_qkv, self.n_g = 2 * H * d + H * dv, H * dv
+        self.proj = ReplicatedLinear(hidden, self.n_qkv + self.n_g + r, dtype=dtype, device=device)
+        self.o_proj = ReplicatedLinear(H * dv, hidden, dtype=dtype, device=device)
+        f = lambda *s: nn.Parameter(torch.zeros(*s, dtype=torch.float32, device=device),  # noqa: E731
+                                    requires_grad=False)
+        self.a2, self.a2_bias = f(H * d, r), f(H * d)
+        self.norm_weight = f(H * dv)            # the shared per-head weight, repeated
+
+    def state_shapes(self) -> tuple:
+        sp = self.spec
+        return ((sp.heads, sp.dim, sp.vdim),)
+
+    def cache_shape(self):
+        return None
+
+    def forward(self, h: torch.Tensor, positions: torch.Tensor, ctx: ForwardContext,
+                cache_idx: int, state: tuple) -> torch.Tensor:
+        sp = self.spec
+        proj = self.proj(h)
+        o = ops.gla_scan(proj, proj[:, self.n_qkv + self.n_g:], self.a2, self.a2_bias, state[0],
+                         ctx.attn, sp.heads, sp.dim, sp.vdim, sp.decay_tau)
+        feats = torch.empty(h.shape[0], self.n_g, dtype=h.dtype, device=h.device)
+        ops.gated_rms_norm(o, proj[:, self.n_qkv: self.n_qkv + self.n_g], self.norm_weight,
+                           sp.heads, self.eps, False, feats)
+        return self.o_proj(feats)
+
+
+class MambaCore(nn.Module):
+    """The selective-scan (Mamba) mixer between its outer projections.  Its projection
+    columns are x | z (``width`` channels each).  x passes a causal convolution with bias and
+    SiLU (the last taps - 1 inputs are per-sequence state); W_x x = dt | B | C (dt_rank, N,
+    N); d = softplus(W_dt dt + dt_bias) per channel; with A = -exp(A_log) [width, N]:
+        S[c, n] = exp(d_c A[c, n]) S[c, n] + d_c x_c B_n,   y_c = S[c, :] . C + D_c x_c
+    (S fp32, per-sequence state); y * silu(z) (times ``out_scale``) is written into a column
+    slice of the output projection's input.  The two inner projections are GEMMs; step
+    sizes, decays and the state are fp32."""
+
+    def __init__(self, spec, eps: float, device, out_scale: float = 1.0, dtype=torch.bfloat16):
+        super().__init__()
+        self.spec, self.out_scale = spec, float(out_scale)
+        I, N, R = spec.width, spec.dim, spec.dt_rank
+        self.n_in, self.n_out = 2 * I, I
+        self.x_proj = ReplicatedLinear(I, R + 2 * N, dtype=dtype, device=device)
+        self.dt_proj = ReplicatedLinear(R, I, dtype=dtype, device=device)
+        f = lambda *s: nn.Parameter(torch.zeros(*s, dtype=torch.float32, device=device),  # noqa: E731
+                                    requires_grad=False)
+        self.conv_w, self.conv_b = f(I, spec.conv), f(I)
+        self.A = f(I, N)                         # -exp(A_log)
+        self.dt_bias, self.dskip = f(I), f(I)
+
+    def state_shapes(self) -> tuple:
+        """Per-slot shapes: the convolution's last inputs, the recurrent state."""
+        sp = self.spec
+        return ((max(sp.conv - 1, 1), sp.width), (sp.width, sp.dim))
+
+    def forward(self, proj: torch.Tensor, col0: int, ctx: ForwardContext, state: tuple,
+                out: torch.Tensor) -> None:
+        sp = self.spec
+        I, R = sp.width, sp.dt_rank
+        x = ops.causal_conv(proj[:, col0: col0 + I], self.conv_w, self.conv_b, state[0],
+                            ctx.attn, True, proj.dtype)
+        dbc = self.x_proj(x)
+        dt = self.dt_proj(dbc[:, :R])
+        ops.selective_scan(x, dt, dbc[:, R:], self.A, self.dt_bias, self.dskip,
+                           proj[:, col0 + I: col0 + 2 * I], state[1], ctx.attn, self.out_scale,
+                           out)

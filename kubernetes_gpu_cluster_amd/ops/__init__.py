@@ -901,11 +901,14 @@ def moe_route_sigmoid(scores: torch.Tensor, correction: torch.Tensor, k: int, sc
 
 
 def grouped_experts(x: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor,
-                    topk_w: torch.Tensor, topk_ids: torch.Tensor, act) -> torch.Tensor:
+                    topk_w: torch.Tensor, topk_ids: torch.Tensor, act,
+                    all_local: bool = True) -> torch.Tensor:
     """sum_j topk_w[t, j] * down_e(act(up_e x[t])), e = topk_ids[t, j], on the grouped MFMA
     GEMM (``moe_align`` buckets, rows gathered for the up projection and scattered back
-    by the down projection, ``moe_combine``): ungated experts w_up [E, I, H], w_down
-    [E, H, I] with the activation ``act`` between.  No host synchronisation."""
+    by the down projection, ``moe_combine``): experts w_up [E, I, H] (gated: [E, 2 I, H],
+    ``act`` halving the columns), w_down [E, H, I] with the activation ``act`` between.
+    ``all_local=False``: ids outside [0, E) are allowed and add nothing.  No host
+    synchronisation."""
     k = _k()
     T, H = x.shape
     E, I = w_up.shape[0], w_up.shape[1]
@@ -922,11 +925,12 @@ def grouped_experts(x: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor,
     k.moe_gemm(inter, x.contiguous(), w_up, sorted_ids, block_expert, meta, npairs, topk, bm,
                True, False)
     a = act(inter)
-    S = moe_splitk(npairs, E, H, I, bm)
+    S = moe_splitk(npairs, E, H, a.shape[1], bm)
+    alloc = torch.empty if all_local else torch.zeros
     if S > 1:
-        y = torch.empty(S, npairs, H, dtype=torch.float32, device=dev)
+        y = alloc(S, npairs, H, dtype=torch.float32, device=dev)
     else:
-        y = torch.empty(npairs, H, dtype=x.dtype, device=dev)
+        y = alloc(npairs, H, dtype=x.dtype, device=dev)
     k.moe_gemm(y, a, w_down, sorted_ids, block_expert, meta, npairs, topk, bm, False, True, S)
     out = torch.empty(T, H, dtype=x.dtype, device=dev)
     k.moe_combine(out, y, topk_w.contiguous().float())
@@ -983,13 +987,15 @@ def side_input(x: torch.Tensor, y: Optional[torch.Tensor], mult: float, gate_w: 
 # with a SiLU gate.  State tensors hold one fp32 entry per sequence slot; a chunk that
 # starts at position 0 starts from zeros, and rows of slot < 0 (graph padding) are skipped.
 def causal_conv(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor],
-                state: torch.Tensor, meta, silu: bool = True) -> torch.Tensor:
-    """fp32 [T, C]: y[t, c] = act(sum_j w[c, j] x[t - (K - 1) + j, c] + bias[c]) per
-    sequence; x [T, C] is a column slice of a projection, w fp32 [C, K], state fp32
-    [slots, K - 1, C] each sequence's last K - 1 inputs (read, then replaced)."""
+                state: torch.Tensor, meta, silu: bool = True,
+                out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+    """[T, C] in ``out_dtype`` (fp32, or x's dtype): y[t, c] = act(sum_j w[c, j]
+    x[t - (K - 1) + j, c] + bias[c]) per sequence; x [T, C] is a column slice of a
+    projection, w fp32 [C, K], state fp32 [slots, K - 1, C] each sequence's last K - 1
+    inputs (read, then replaced)."""
     if not _gpu(x):
-        return ref.causal_conv(x, w, bias, state, ref.step_sequences(meta), silu)
-    out = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+        return ref.causal_conv(x, w, bias, state, ref.step_sequences(meta), silu, out_dtype)
+    out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
     ws, wb = getattr(meta, "work_seq", None), getattr(meta, "work_mblk", None)
     if meta.num_prefills and ws is None:
         qsl = meta.query_start_loc.tolist()
@@ -1047,3 +1053,101 @@ def gated_rms_norm(y: torch.Tensor, gate: torch.Tensor, w: torch.Tensor, groups:
         return out
     _k().gated_rms_norm(out, y, gate, w, groups, eps, gate_first)
     return out
+
+
+# ------------------------------------------------------------------ Lorenex-style decoders
+# Gated linear attention with a decay per key channel and the selective scan over
+# per-sequence state slots, attention inputs made unit-RMS vectors with a position-dependent
+# query factor, PolyNorm, clamped gated experts, softmax routing over all router outputs
+# with a choice correction and identity experts.
+def embed_pos(ids: torch.Tensor, positions: torch.Tensor, table: torch.Tensor, scale: float,
+              pos_table: Optional[torch.Tensor], out: torch.Tensor) -> torch.Tensor:
+    """out fp32 [T, W] = table[ids] * scale (+ pos_table[positions]): the start of an fp32
+    residual stream with a scaled embedding and learned positions."""
+    if not _gpu(out):
+        return ref.embed_pos(ids, positions, table, scale, pos_table, out)
+    _k().embed_pos(out, ids, positions, table, pos_table, float(scale))
+    return out
+
+
+def gla_scan(proj: torch.Tensor, low: torch.Tensor, a2: torch.Tensor, a2_bias: torch.Tensor,
+             state: torch.Tensor, meta, H: int, d: int, dv: int, tau: float) -> torch.Tensor:
+    """fp32 [T, H dv]: gated linear attention over every step sequence's rows from / into
+    state [slots, H, d, dv]; proj [T, >= 2 H d + H dv] = q | k | v, low [T, r] (a column slice)
+    the decay bottleneck, a2 fp32 [H d, r], a2_bias fp32 [H d]; see ``ref.gla_scan``."""
+    if not _gpu(proj):
+        return ref.gla_scan(proj, low, a2, a2_bias, state, ref.step_sequences(meta), H, d, dv, tau)
+    out = torch.empty(proj.shape[0], H * dv, dtype=torch.float32, device=proj.device)
+    _k().gla_scan(out, proj, low, a2, a2_bias, state, meta.query_start_loc,
+                  meta.prefill_seq_lens, meta.decode_ctx_lens, meta.state_slots,
+                  meta.num_prefills, meta.num_decodes, meta.num_prefill_tokens, H, d, dv,
+                  float(tau))
+    return out
+
+
+def selective_scan(x: torch.Tensor, dt: torch.Tensor, bc: torch.Tensor, A: torch.Tensor,
+                   dt_bias: torch.Tensor, dskip: torch.Tensor, z: torch.Tensor,
+                   state: torch.Tensor, meta, out_scale: float, out: torch.Tensor) -> torch.Tensor:
+    """out [T, I] (a column slice of a wider buffer) = y * silu(z) * out_scale, y the
+    selective scan over every step sequence's rows from / into state [slots, I, N]; x, dt
+    [T, I], bc [T, 2 N] and z [T, I] (column slices), A fp32 [I, N]; see
+    ``ref.selective_scan``."""
+    if not _gpu(x):
+        out.copy_(ref.selective_scan(x, dt, bc, A, dt_bias, dskip, z, state,
+                                     ref.step_sequences(meta), out_scale, out.dtype))
+        return out
+    _k().selective_scan(out, x, dt, bc, A, dt_bias, dskip, z, state, meta.query_start_loc,
+                        meta.prefill_seq_lens, meta.decode_ctx_lens, meta.state_slots,
+                        meta.num_prefills, meta.num_decodes, meta.num_prefill_tokens,
+                        float(out_scale))
+    return out
+
+
+def norm_kv_store(qkv: torch.Tensor, positions: torch.Tensor, k_cache: torch.Tensor,
+                  v_cache: torch.Tensor, slot_mapping: torch.Tensor, H: int, G: int, dk: int,
+                  dv: int, eps: float, qk_unit: bool, v_unit: bool, q_temp,
+                  out_dtype: torch.dtype) -> torch.Tensor:
+    """q [T, H, dk] in ``out_dtype`` from qkv fp32 [T, H dk + G dk + G dv], k and v into the
+    paged cache: head vectors divided by their root mean square (``qk_unit``, ``v_unit``),
+    q times 1 + coef * ln(floor((p + 1) / every) + 1) (``q_temp`` = (coef, every) or None)."""
+    if not _gpu(qkv):
+        return ref.norm_kv_store(qkv, positions, k_cache, v_cache, slot_mapping, H, G, dk, dv,
+                                 eps, qk_unit, v_unit, q_temp, out_dtype)
+    q = torch.empty(qkv.shape[0], H, dk, dtype=out_dtype, device=qkv.device)
+    coef, every = q_temp if q_temp is not None else (0.0, 1)
+    _k().norm_kv_store(qkv, positions, q, k_cache, v_cache, slot_mapping, H, G, dk, dv,
+                       float(eps), qk_unit, v_unit, float(coef), int(every))
+    return q
+
+
+def polynorm(z: torch.Tensor, coef: torch.Tensor, eps: float) -> torch.Tensor:
+    """a N(z) + b N(z^2) + c N(z^3) + e per row of z [T, F], coef fp32 [4]."""
+    if not _gpu(z):
+        return ref.polynorm(z, coef, eps)
+    out = torch.empty_like(z)
+    _k().polynorm(out, z, coef, float(eps))
+    return out
+
+
+def swiglu_clamp(x: torch.Tensor, limit: float, alpha: float = 1.702) -> torch.Tensor:
+    """x [..., 2 I] = gate | up -> min(gate, limit) sigmoid(alpha .) (clamp(up, +-limit) + 1)."""
+    if not _gpu(x):
+        return ref.swiglu_clamp(x, limit, alpha)
+    I = x.shape[-1] // 2
+    x2 = x.reshape(-1, 2 * I)
+    out = torch.empty(x2.shape[0], I, dtype=x.dtype, device=x.device)
+    _k().swiglu_clamp(out, x2, float(limit), float(alpha))
+    return out.view(*x.shape[:-1], I)
+
+
+def moe_route_softmax_all(logits: torch.Tensor, correction: torch.Tensor, k: int, n_real: int):
+    """(weights fp32 [T, k], expert ids int32 [T, k], identity weight fp32 [T]) from router
+    logits fp32 [T, >= E]; see ``ref.moe_route_softmax_all``."""
+    if not _gpu(logits):
+        return ref.moe_route_softmax_all(logits, correction, k, n_real)
+    T = logits.shape[0]
+    w = torch.empty(T, k, dtype=torch.float32, device=logits.device)
+    ids = torch.empty(T, k, dtype=torch.int32, device=logits.device)
+    idw = torch.empty(T, dtype=torch.float32, device=logits.device)
+    _k().moe_route_softmax_all(w, ids, idw, logits, correction, int(n_real))
+    return w, ids, idw

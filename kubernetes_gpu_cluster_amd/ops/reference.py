@@ -708,7 +708,9 @@ def moe_finish(routed: Optional[torch.Tensor], dense: Optional[torch.Tensor],
         out = routed.float()
     else:
         T = dense.shape[1]
-        y = dense.float()[topk_ids.long(), torch.arange(T, device=dense.device)[:, None]]
+        ids = topk_ids.long()
+        ids = torch.where((ids < 0) | (ids >= dense.shape[0]), torch.zeros_like(ids), ids)
+        y = dense.float()[ids, torch.arange(T, device=dense.device)[:, None]]
         out = (y * topk_w.float()[:, :, None]).sum(1)
     if shared is not None:
         out = out + gate.float()[:, None] * shared.float()
@@ -727,11 +729,13 @@ def side_gate(pre: torch.Tensor, ids: torch.Tensor, table: torch.Tensor, col0: i
 # (short causal convolutions over per-sequence state, the Mamba-2 recurrence, the gated
 # delta rule, RMS norms combined with a SiLU gate)
 def causal_conv(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor],
-                state: torch.Tensor, seqs: list, silu: bool = True) -> torch.Tensor:
+                state: torch.Tensor, seqs: list, silu: bool = True,
+                out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
     """Per-channel causal convolution over time: y[t, c] = sum_j w[c, j] * x[t - (K-1) + j, c]
     (+ bias[c]), the last tap on the current token, then SiLU.  x [T, C] (a column slice of
     a projection), w fp32 [C, K].  state fp32 [slots, K-1, C] holds each sequence's last
-    K-1 inputs (oldest first; zeros before position 0) and is updated.  -> fp32 [T, C]."""
+    K-1 inputs (oldest first; zeros before position 0) and is updated.  -> [T, C] in
+    ``out_dtype`` (fp32 math)."""
     T, C = x.shape
     K = w.shape[1]
     out = torch.zeros(T, C, dtype=torch.float32, device=x.device)
@@ -749,7 +753,7 @@ def causal_conv(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor],
         out[a:a + n] = y
         if K > 1:
             state[slot] = xs[n:]
-    return out * torch.sigmoid(out) if silu else out
+    return (out * torch.sigmoid(out) if silu else out).to(out_dtype)
 
 
 def ssd_scan(xbc: torch.Tensor, dt: torch.Tensor, a_log: torch.Tensor, dt_bias: torch.Tensor,
@@ -823,3 +827,137 @@ def gated_rms_norm(y: torch.Tensor, gate: torch.Tensor, w: torch.Tensor, groups:
     vg = v.view(T, groups, n // groups)
     v = (vg * torch.rsqrt(vg.pow(2).mean(-1, keepdim=True) + eps)).view(T, n) * w.float()
     return (v if gate_first else v * g).to(out_dtype)
+
+
+# ---------------------------------------------------------------- Lorenex-style decoders
+# (gated linear attention with a decay per key channel, the selective scan, attention inputs
+# made unit-RMS vectors with a position-dependent query factor, PolyNorm, clamped gated
+# experts, softmax routing over all router outputs with a choice correction)
+def embed_pos(ids: torch.Tensor, positions: torch.Tensor, table: torch.Tensor, scale: float,
+              pos_table: Optional[torch.Tensor], out: torch.Tensor) -> torch.Tensor:
+    """out fp32 [T, W] = table[ids] * scale (+ pos_table[positions])."""
+    x = table[ids.long()].float() * scale
+    if pos_table is not None:
+        x = x + pos_table[positions.long().clamp(0, pos_table.shape[0] - 1)].float()
+    out.copy_(x)
+    return out
+
+
+def gla_scan(proj: torch.Tensor, low: torch.Tensor, a2: torch.Tensor, a2_bias: torch.Tensor,
+             state: torch.Tensor, seqs: list, H: int, d: int, dv: int, tau: float) -> torch.Tensor:
+    """Gated linear attention.  proj [T, >= 2 H d + H dv] = q | k | v (| ...); low [T, r] the
+    decay bottleneck; a2 fp32 [H d, r], a2_bias fp32 [H d].  Per head, with
+    ln alpha = logsigmoid(a2 low + a2_bias) / tau (one decay per key channel) and q times
+    d^-1/2:   S = diag(alpha) S + k v^T;  o = S^T q      (S [d, dv])
+    from state[slot] [H, d, dv] fp32 (zeros at position 0), written back.  -> fp32 [T, H dv]."""
+    T = proj.shape[0]
+    q = proj[:, : H * d].float().view(T, H, d) * d ** -0.5
+    k = proj[:, H * d: 2 * H * d].float().view(T, H, d)
+    v = proj[:, 2 * H * d: 2 * H * d + H * dv].float().view(T, H, dv)
+    z = low.float() @ a2.float().t() + a2_bias.float()
+    alpha = torch.exp(torch.nn.functional.logsigmoid(z) / tau).view(T, H, d)
+    out = torch.zeros(T, H, dv, dtype=torch.float32)
+    for a, n, p0, slot in seqs:
+        if slot < 0:
+            continue
+        S = torch.zeros(H, d, dv) if p0 == 0 else state[slot].clone()
+        for t in range(a, a + n):
+            S = alpha[t][:, :, None] * S + k[t][:, :, None] * v[t][:, None, :]
+            out[t] = torch.einsum("hdv,hd->hv", S, q[t])
+        state[slot] = S
+    return out.view(T, H * dv)
+
+
+def selective_scan(x: torch.Tensor, dt: torch.Tensor, bc: torch.Tensor, A: torch.Tensor,
+                   dt_bias: torch.Tensor, dskip: torch.Tensor, z: torch.Tensor,
+                   state: torch.Tensor, seqs: list, out_scale: float,
+                   out_dtype: torch.dtype) -> torch.Tensor:
+    """The selective scan.  x [T, I] (after convolution and SiLU), dt [T, I] raw step sizes,
+    bc [T, 2 N] = B | C, A fp32 [I, N] (negative), z [T, I] the gate pre-activation.  With
+    d = softplus(dt + dt_bias), per channel c and state n:
+        S[c, n] = exp(d_c A[c, n]) S[c, n] + d_c x_c B_n;   y_c = sum_n S[c, n] C_n + dskip_c x_c
+    from state[slot] [I, N] fp32 (zeros at position 0), written back.
+    -> y * silu(z) * out_scale in out_dtype [T, I]."""
+    T, I = x.shape
+    N = A.shape[1]
+    xf = x.float()
+    d = torch.nn.functional.softplus(dt.float() + dt_bias.float())
+    B, C = bc[:, :N].float(), bc[:, N: 2 * N].float()
+    y = torch.zeros(T, I, dtype=torch.float32)
+    for a, n, p0, slot in seqs:
+        if slot < 0:
+            continue
+        S = torch.zeros(I, N) if p0 == 0 else state[slot].clone()
+        for t in range(a, a + n):
+            S = torch.exp(d[t][:, None] * A.float()) * S + (d[t] * xf[t])[:, None] * B[t][None, :]
+            y[t] = S @ C[t] + dskip.float() * xf[t]
+        state[slot] = S
+    zf = z.float()
+    return (y * (zf * torch.sigmoid(zf)) * out_scale).to(out_dtype)
+
+
+def norm_kv_store(qkv: torch.Tensor, positions: torch.Tensor, k_cache: torch.Tensor,
+                  v_cache: torch.Tensor, slot_mapping: torch.Tensor, H: int, G: int, dk: int,
+                  dv: int, eps: float, qk_unit: bool, v_unit: bool, q_temp,
+                  out_dtype: torch.dtype) -> torch.Tensor:
+    """qkv fp32 [T, H dk + G dk + G dv] -> q [T, H, dk] in out_dtype; k and v go to the
+    plain-layout paged cache at ``slot_mapping`` (< 0: no write).  ``qk_unit`` / ``v_unit``:
+    each head's vector is divided by sqrt(mean(x^2) + eps).  ``q_temp`` = (coef, every): q at
+    position p times 1 + coef * ln(floor((p + 1) / every) + 1).  fp32 math."""
+    T = qkv.shape[0]
+    q = qkv[:, : H * dk].float().view(T, H, dk)
+    k = qkv[:, H * dk: (H + G) * dk].float().view(T, G, dk)
+    v = qkv[:, (H + G) * dk: (H + G) * dk + G * dv].float().view(T, G, dv)
+
+    def unit(x):
+        return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+    if qk_unit:
+        q, k = unit(q), unit(k)
+    if v_unit:
+        v = unit(v)
+    if q_temp is not None:
+        coef, every = q_temp
+        p = positions.clamp(min=0)
+        f = 1.0 + coef * torch.log((torch.div(p + 1, every, rounding_mode="floor") + 1).float())
+        q = q * f[:, None, None]
+    bs = k_cache.shape[2]
+    ok = slot_mapping >= 0
+    sl = slot_mapping[ok].long()
+    k_cache[sl // bs, :, sl % bs] = k[ok].to(k_cache.dtype)
+    v_cache[sl // bs, :, sl % bs] = v[ok].to(v_cache.dtype)
+    return q.to(out_dtype)
+
+
+def polynorm(z: torch.Tensor, coef: torch.Tensor, eps: float) -> torch.Tensor:
+    """a N(z) + b N(z^2) + c N(z^3) + e over rows of z [T, F]: powers element by element,
+    N(v) = v / sqrt(mean(v^2) + eps), coef fp32 [4] = (a, b, c, e).  fp32 math."""
+    zf = z.float()
+
+    def n(v):
+        return v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps)
+    c = coef.float()
+    return (c[0] * n(zf) + c[1] * n(zf * zf) + c[2] * n(zf * zf * zf) + c[3]).to(z.dtype)
+
+
+def swiglu_clamp(x: torch.Tensor, limit: float, alpha: float = 1.702) -> torch.Tensor:
+    """x [rows, 2 I] = gate | up  ->  g sigmoid(alpha g) (u + 1) with g = min(gate, limit),
+    u = clamp(up, -limit, limit)."""
+    I = x.shape[-1] // 2
+    g = x[..., :I].float().clamp(max=limit)
+    u = x[..., I:].float().clamp(-limit, limit)
+    return (g * torch.sigmoid(alpha * g) * (u + 1.0)).to(x.dtype)
+
+
+def moe_route_softmax_all(logits: torch.Tensor, correction: torch.Tensor, k: int, n_real: int):
+    """logits fp32 [T, E]: s = softmax over all E router outputs; the k outputs with the
+    largest s + correction are chosen (lowest index first among equals) and weighted by s as
+    it is.  Outputs >= n_real name identity experts: their pairs get weight 0 here and their
+    scores are summed per token.  -> (weights fp32 [T, k], ids int32 [T, k], identity weight
+    fp32 [T])."""
+    E = correction.numel()
+    s = torch.softmax(logits[:, :E].float(), dim=-1)
+    ids = torch.topk(s + correction.float(), k, dim=-1).indices
+    w = torch.gather(s, 1, ids)
+    ident = ids >= n_real
+    idw = (w * ident).sum(-1)
+    return w.masked_fill(ident, 0.0), ids.to(torch.int32), idw
