@@ -1538,11 +1538,13 @@ void causal_conv(Tensor out, Tensor x, Tensor w, std::optional<Tensor> bias, Ten
                  std::optional<Tensor> ctx_lens, Tensor slots, std::optional<Tensor> work_seq,
                  std::optional<Tensor> work_blk, int64_t P, int64_t D, int64_t Tp, bool silu) {
   check_gpu(x, "x");
-  check_f32(out, "out");
+  check_gpu(out, "out");
   check_f32(w, "w");
   check_f32(state, "state");
   c10::hip::HIPGuardMasqueradingAsCUDA g(x.device());
   TORCH_CHECK(x.dim() == 2, "kgc.causal_conv: x [T, C]");
+  TORCH_CHECK(out.device() == x.device() && (out.scalar_type() == at::kFloat ||
+              out.scalar_type() == x.scalar_type()), "kgc.causal_conv: out fp32 or x's dtype");
   const int64_t T = x.size(0), C = x.size(1);
   check_cols(x, T, C, x, "x");
   check_step("causal_conv", T, P, D, Tp);
@@ -1564,7 +1566,8 @@ void causal_conv(Tensor out, Tensor x, Tensor w, std::optional<Tensor> bias, Ten
     wsp = work_seq->data_ptr<int>();
     wbp = work_blk->data_ptr<int>();
   }
-  kgc::launch_causal_conv(dt_code(x), out.data_ptr<float>(), x.data_ptr(), x.stride(0),
+  kgc::launch_causal_conv(dt_code(x), out.data_ptr(), out.scalar_type() == at::kFloat,
+                          x.data_ptr(), x.stride(0),
                           w.data_ptr<float>(), f32_opt(bias, C, "bias"), state.data_ptr<float>(),
                           i32_ptr(qsl, P ? P + 1 : 0, "query_start_loc"),
                           i32_ptr(seq_lens, P, "seq_lens"), i32_ptr(ctx_lens, D, "ctx_lens"),
@@ -1643,6 +1646,177 @@ void gated_rms_norm(Tensor out, Tensor y, Tensor gate, Tensor w, int64_t groups,
   kgc::launch_gated_rms_norm(dt_code(gate), out.data_ptr(), out.stride(0), y.data_ptr<float>(),
                              gate.data_ptr(), gate.stride(0), f32_opt(w, n, "w"), (int)T, (int)n,
                              (int)groups, (float)eps, gate_first, stream());
+}
+
+// ---- gated linear attention, selective scan, unit-RMS attention inputs, PolyNorm, clamped
+// ---- gated activation, softmax routing over all outputs, scaled embedding + positions ------
+void gla_scan(Tensor out, Tensor proj, Tensor low, Tensor a2, Tensor a2_bias, Tensor S,
+              std::optional<Tensor> qsl, std::optional<Tensor> seq_lens,
+              std::optional<Tensor> ctx_lens, Tensor slots, int64_t P, int64_t D, int64_t Tp,
+              int64_t H, int64_t d, int64_t V, double tau) {
+  check_gpu(proj, "proj");
+  check_f32(out, "out");
+  check_f32(S, "S");
+  c10::hip::HIPGuardMasqueradingAsCUDA g(proj.device());
+  TORCH_CHECK(H >= 1 && H <= 65535 && V >= 1 && d >= 1 && d <= kgc::decay_scan_max_rows() &&
+              tau > 0, "kgc.gla_scan: head sizes / tau");
+  TORCH_CHECK(proj.dim() == 2 && proj.stride(1) == 1 && act_dtype(proj) &&
+              proj.size(1) >= 2 * H * d + H * V, "kgc.gla_scan: proj [T, >= 2 H d + H V]");
+  const int64_t T = proj.size(0);
+  check_step("gla_scan", T, P, D, Tp);
+  TORCH_CHECK(low.dim() == 2 && low.size(1) >= 1 && low.size(1) <= kgc::gla_scan_max_rank(),
+              "kgc.gla_scan: low [T, rank <= 128]");
+  const int64_t R = low.size(1);
+  check_cols(low, T, R, proj, "low");
+  TORCH_CHECK(low.scalar_type() == proj.scalar_type(), "kgc.gla_scan: low / proj dtypes");
+  TORCH_CHECK(a2.is_contiguous() && a2.dim() == 2 && a2.size(0) == H * d && a2.size(1) == R &&
+              a2.device() == proj.device(), "kgc.gla_scan: a2 [H d, rank]");
+  TORCH_CHECK(out.is_contiguous() && out.numel() == T * H * V && out.device() == proj.device(),
+              "kgc.gla_scan: out [T, H V]");
+  TORCH_CHECK(S.is_contiguous() && S.dim() == 4 && S.size(1) == H && S.size(2) == d &&
+              S.size(3) == V && S.device() == proj.device(), "kgc.gla_scan: state [slots, H, d, V]");
+  kgc::launch_gla_scan(dt_code(proj), out.data_ptr<float>(), proj.data_ptr(), proj.stride(0),
+                       low.data_ptr(), low.stride(0), f32_opt(a2, H * d * R, "a2"),
+                       f32_opt(a2_bias, H * d, "a2_bias"), S.data_ptr<float>(),
+                       i32_ptr(qsl, P ? P + 1 : 0, "query_start_loc"),
+                       i32_ptr(seq_lens, P, "seq_lens"), i32_ptr(ctx_lens, D, "ctx_lens"),
+                       i32_ptr(slots, P + D, "state slots"), (int)P, (int)D, (int)Tp, (int)H,
+                       (int)d, (int)V, (int)R, (float)tau, (int)S.size(0), stream());
+}
+
+void selective_scan(Tensor out, Tensor x, Tensor dt, Tensor bc, Tensor At, Tensor dt_bias,
+                    Tensor dskip, Tensor z, Tensor S, std::optional<Tensor> qsl,
+                    std::optional<Tensor> seq_lens, std::optional<Tensor> ctx_lens, Tensor slots,
+                    int64_t P, int64_t D, int64_t Tp, double out_scale) {
+  check_gpu(x, "x");
+  check_f32(S, "S");
+  c10::hip::HIPGuardMasqueradingAsCUDA g(x.device());
+  TORCH_CHECK(x.dim() == 2 && x.is_contiguous() && act_dtype(x), "kgc.selective_scan: x [T, I]");
+  const int64_t T = x.size(0), I = x.size(1);
+  check_step("selective_scan", T, P, D, Tp);
+  TORCH_CHECK(At.dim() == 2 && At.is_contiguous() && At.size(1) == I && At.size(0) >= 1 &&
+              At.size(0) <= kgc::decay_scan_max_rows() && At.device() == x.device(),
+              "kgc.selective_scan: At [N <= 256, I]");
+  const int64_t N = At.size(0);
+  TORCH_CHECK(dt.is_contiguous() && dt.dim() == 2 && dt.size(0) == T && dt.size(1) == I &&
+              dt.scalar_type() == x.scalar_type() && dt.device() == x.device(),
+              "kgc.selective_scan: dt [T, I]");
+  check_cols(bc, T, 2 * N, x, "bc");
+  check_cols(z, T, I, x, "z");
+  check_cols(out, T, I, x, "out");
+  TORCH_CHECK(bc.scalar_type() == x.scalar_type() && z.scalar_type() == x.scalar_type() &&
+              out.scalar_type() == x.scalar_type(), "kgc.selective_scan: dtypes");
+  TORCH_CHECK(S.is_contiguous() && S.dim() == 3 && S.size(1) == N && S.size(2) == I &&
+              S.device() == x.device(), "kgc.selective_scan: state [slots, N, I]");
+  kgc::launch_selective_scan(dt_code(x), out.data_ptr(), out.stride(0), x.data_ptr(),
+                             dt.data_ptr(), bc.data_ptr(), bc.stride(0),
+                             f32_opt(At, N * I, "At"), f32_opt(dt_bias, I, "dt_bias"),
+                             f32_opt(dskip, I, "dskip"), z.data_ptr(), z.stride(0),
+                             S.data_ptr<float>(), i32_ptr(qsl, P ? P + 1 : 0, "query_start_loc"),
+                             i32_ptr(seq_lens, P, "seq_lens"), i32_ptr(ctx_lens, D, "ctx_lens"),
+                             i32_ptr(slots, P + D, "state slots"), (int)P, (int)D, (int)Tp,
+                             (int)I, (int)N, (float)out_scale, (int)S.size(0), stream());
+}
+
+void norm_kv_store(Tensor qkv, Tensor positions, Tensor q_out, Tensor k_cache, Tensor v_cache,
+                   Tensor slots, int64_t H, int64_t G, int64_t dk, int64_t dv, double eps,
+                   bool qk_unit, bool v_unit, double coef, int64_t every) {
+  check_gpu(qkv, "qkv");
+  check_f32(qkv, "qkv");
+  c10::hip::HIPGuardMasqueradingAsCUDA g(qkv.device());
+  TORCH_CHECK(qkv.dim() == 2 && qkv.stride(1) == 1 && qkv.size(1) >= (H + G) * dk + G * dv &&
+              H >= 1 && G >= 1 && dk >= 1 && dv >= 1 && every >= 1,
+              "kgc.norm_kv_store: qkv fp32 [T, H dk + G dk + G dv]");
+  const int64_t T = qkv.size(0);
+  TORCH_CHECK(q_out.is_cuda() && q_out.device() == qkv.device() && act_dtype(q_out) &&
+              q_out.is_contiguous() && q_out.numel() == T * H * dk, "kgc.norm_kv_store: q_out");
+  check_plain_cache(k_cache, v_cache, q_out, G, dk, dv);
+  TORCH_CHECK(positions.scalar_type() == at::kLong && positions.numel() == T &&
+              positions.is_contiguous() && slots.scalar_type() == at::kLong &&
+              slots.numel() == T && slots.is_contiguous() && positions.is_cuda() && slots.is_cuda(),
+              "kgc.norm_kv_store: positions / slots int64 [T]");
+  kgc::launch_norm_kv_store(dt_code(q_out), qkv.data_ptr<float>(), qkv.stride(0),
+                            positions.data_ptr<int64_t>(), q_out.data_ptr(), k_cache.data_ptr(),
+                            v_cache.data_ptr(), slots.data_ptr<int64_t>(), (int)T, (int)H, (int)G,
+                            (int)dk, (int)dv, (int)k_cache.size(2), (int)k_cache.size(0),
+                            (float)eps, qk_unit, v_unit, (float)coef, (int)every, stream());
+}
+
+void polynorm(Tensor out, Tensor z, Tensor coef, double eps) {
+  check_gpu(z, "z");
+  c10::hip::HIPGuardMasqueradingAsCUDA g(z.device());
+  TORCH_CHECK(z.dim() == 2 && z.is_contiguous() && act_dtype(z) && out.is_contiguous() &&
+              out.sizes() == z.sizes() && out.scalar_type() == z.scalar_type() &&
+              out.device() == z.device(), "kgc.polynorm: z, out [rows, F]");
+  TORCH_CHECK(coef.device() == z.device(), "kgc.polynorm: coef device");
+  kgc::launch_polynorm(dt_code(z), out.data_ptr(), z.data_ptr(), f32_opt(coef, 4, "coef"),
+                       z.size(0), (int)z.size(1), (float)eps, stream());
+}
+
+void swiglu_clamp(Tensor out, Tensor x, double limit, double alpha) {
+  check_gpu(x, "x");
+  c10::hip::HIPGuardMasqueradingAsCUDA g(x.device());
+  TORCH_CHECK(x.dim() == 2 && x.is_contiguous() && act_dtype(x) && x.size(1) % 2 == 0 &&
+              out.is_contiguous() && out.dim() == 2 && out.size(0) == x.size(0) &&
+              out.size(1) * 2 == x.size(1) && out.scalar_type() == x.scalar_type() &&
+              out.device() == x.device(), "kgc.swiglu_clamp: x [rows, 2 I], out [rows, I]");
+  kgc::launch_swiglu_clamp(dt_code(x), out.data_ptr(), x.data_ptr(), x.size(0), (int)out.size(1),
+                           (float)limit, (float)alpha, stream());
+}
+
+void embed_pos(Tensor out, Tensor ids, Tensor positions, Tensor table,
+               std::optional<Tensor> pos_table, double scale) {
+  check_gpu(out, "out");
+  check_f32(out, "out");
+  c10::hip::HIPGuardMasqueradingAsCUDA g(out.device());
+  TORCH_CHECK(out.dim() == 2 && out.is_contiguous(), "kgc.embed_pos: out [T, W]");
+  const int64_t T = out.size(0), W = out.size(1);
+  TORCH_CHECK(table.is_cuda() && table.device() == out.device() && table.dim() == 2 &&
+              table.is_contiguous() && table.size(1) == W && act_dtype(table),
+              "kgc.embed_pos: table [vocab, W]");
+  TORCH_CHECK(ids.scalar_type() == at::kLong && ids.numel() == T && ids.is_contiguous() &&
+              positions.scalar_type() == at::kLong && positions.numel() == T &&
+              positions.is_contiguous() && ids.is_cuda() && positions.is_cuda(),
+              "kgc.embed_pos: ids / positions int64 [T]");
+  const float* pp = nullptr;
+  int64_t max_pos = 0;
+  if (pos_table.has_value()) {
+    check_f32(*pos_table, "pos_table");
+    TORCH_CHECK(pos_table->dim() == 2 && pos_table->is_contiguous() && pos_table->size(1) == W &&
+                pos_table->size(0) >= 1 && pos_table->device() == out.device(),
+                "kgc.embed_pos: pos_table fp32 [max_pos, W]");
+    pp = pos_table->data_ptr<float>();
+    max_pos = pos_table->size(0);
+  }
+  kgc::launch_embed_pos(dt_code(table), out.data_ptr<float>(), ids.data_ptr<int64_t>(),
+                        positions.data_ptr<int64_t>(), table.data_ptr(), pp, (int)T, (int)W,
+                        (int)table.size(0), (int)max_pos, (float)scale, stream());
+}
+
+void moe_route_softmax_all(Tensor w, Tensor ids, Tensor idw, Tensor logits, Tensor correction,
+                           int64_t n_real) {
+  check_gpu(logits, "logits");
+  check_f32(logits, "logits");
+  check_f32(w, "w");
+  check_f32(idw, "idw");
+  c10::hip::HIPGuardMasqueradingAsCUDA g(logits.device());
+  TORCH_CHECK(logits.dim() == 2 && logits.stride(1) == 1 && logits.device() == w.device(),
+              "kgc.moe_route_softmax_all: logits fp32 [T, >= E]");
+  const int64_t T = logits.size(0), E = correction.numel();
+  TORCH_CHECK(w.dim() == 2 && w.size(0) == T && w.is_contiguous(), "kgc.moe_route_softmax_all: w [T, k]");
+  const int64_t k = w.size(1);
+  TORCH_CHECK(E >= 1 && E <= logits.size(1) && E <= kgc::moe_route_sigmoid_max_experts() &&
+              k >= 1 && k <= E && k <= 64 && n_real >= 0 && n_real <= E,
+              "kgc.moe_route_softmax_all: experts / top");
+  TORCH_CHECK(ids.is_cuda() && ids.scalar_type() == at::kInt && ids.is_contiguous() &&
+              ids.numel() == T * k && ids.device() == w.device() && idw.is_contiguous() &&
+              idw.numel() == T && idw.device() == w.device(),
+              "kgc.moe_route_softmax_all: ids int32 [T, k], idw fp32 [T]");
+  TORCH_CHECK(correction.device() == w.device(), "kgc.moe_route_softmax_all: correction device");
+  kgc::launch_moe_route_softmax_all(w.data_ptr<float>(), ids.data_ptr<int>(),
+                                    idw.data_ptr<float>(), logits.data_ptr<float>(),
+                                    logits.stride(0), f32_opt(correction, E, "correction"),
+                                    (int)T, (int)E, (int)k, (int)n_real, stream());
 }
 
 void residual_norm(std::optional<Tensor> out, Tensor x, std::optional<Tensor> add,
@@ -1924,6 +2098,21 @@ void moe_finish(Tensor out, std::optional<Tensor> routed, std::optional<Tensor> 
 }  // namespace
 
 TORCH_LIBRARY(kgc, m) {
+  m.def("gla_scan(Tensor(a!) out, Tensor proj, Tensor low, Tensor a2, Tensor a2_bias, Tensor(b!) S, "
+        "Tensor? qsl, Tensor? seq_lens, Tensor? ctx_lens, Tensor slots, int P, int D, int Tp, int H, "
+        "int d, int V, float tau) -> ()");
+  m.def("selective_scan(Tensor(a!) out, Tensor x, Tensor dt, Tensor bc, Tensor At, Tensor dt_bias, "
+        "Tensor dskip, Tensor z, Tensor(b!) S, Tensor? qsl, Tensor? seq_lens, Tensor? ctx_lens, "
+        "Tensor slots, int P, int D, int Tp, float out_scale) -> ()");
+  m.def("norm_kv_store(Tensor qkv, Tensor positions, Tensor(a!) q_out, Tensor(b!) k_cache, "
+        "Tensor(c!) v_cache, Tensor slots, int H, int G, int dk, int dv, float eps, bool qk_unit, "
+        "bool v_unit, float coef, int every) -> ()");
+  m.def("polynorm(Tensor(a!) out, Tensor z, Tensor coef, float eps) -> ()");
+  m.def("swiglu_clamp(Tensor(a!) out, Tensor x, float limit, float alpha) -> ()");
+  m.def("embed_pos(Tensor(a!) out, Tensor ids, Tensor positions, Tensor table, Tensor? pos_table, "
+        "float scale) -> ()");
+  m.def("moe_route_softmax_all(Tensor(a!) w, Tensor(b!) ids, Tensor(c!) idw, Tensor logits, "
+        "Tensor correction, int n_real) -> ()");
   m.def("residual_norm(Tensor(a!)? out, Tensor(b!) x, Tensor? add, Tensor? add_norm_w, Tensor? w, "
         "float mult, float eps) -> ()");
   m.def("token_shift(Tensor(a!) out, Tensor h, Tensor mu, Tensor(b!) state, Tensor? qsl, Tensor? seq_lens, "
@@ -2075,6 +2264,13 @@ TORCH_LIBRARY(kgc, m) {
 }
 
 TORCH_LIBRARY_IMPL(kgc, CUDA, m) {
+  m.impl("gla_scan", &gla_scan);
+  m.impl("selective_scan", &selective_scan);
+  m.impl("norm_kv_store", &norm_kv_store);
+  m.impl("polynorm", &polynorm);
+  m.impl("swiglu_clamp", &swiglu_clamp);
+  m.impl("embed_pos", &embed_pos);
+  m.impl("moe_route_softmax_all", &moe_route_softmax_all);
   m.impl("residual_group_norm", &residual_group_norm);
   m.impl("depth_mix_norm", &depth_mix_norm);
   m.impl("head_norm_gate", &head_norm_gate);

@@ -67,6 +67,44 @@ __global__ __launch_bounds__(256) void rope_kv_store_kernel(
   }
 }
 
+// Attention inputs as unit-RMS vectors: qkv fp32 [T, H dk + G dk + G dv] (row stride qs).
+// Each head's q and k (qk_unit) and v (v_unit) is divided by sqrt(mean(x^2) + eps); q at
+// position p is multiplied by 1 + coef * ln(floor((p + 1) / every) + 1); q goes to q_out
+// [T, H, dk], k and v into the cache.  One wave per head vector, fp32 math.
+template <typename T>
+__global__ __launch_bounds__(256) void norm_kv_store_kernel(
+    const float* __restrict__ qkv, int64_t qs, const int64_t* __restrict__ positions,
+    T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache,
+    const int64_t* __restrict__ slots, int H, int G, int dk, int dv, int bs, int num_blocks,
+    float eps, bool qk_unit, bool v_unit, float coef, int every) {
+  const int64_t t = blockIdx.x;
+  const float* row = qkv + t * qs;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  int64_t pos = positions[t];
+  if (pos < 0) pos = 0;
+  const float temp = coef != 0.f ? 1.f + coef * logf((float)((pos + 1) / every) + 1.f) : 1.f;
+  const int64_t slot = slots[t];
+  const bool store = slot >= 0 && slot < (int64_t)num_blocks * bs;
+  const int64_t blk = store ? slot / bs : 0, off = store ? slot % bs : 0;
+  for (int hv = wave; hv < H + 2 * G; hv += 4) {
+    const bool isq = hv < H, isk = !isq && hv < H + G;
+    const int n = hv < H + G ? dk : dv;
+    const float* src = row + (hv < H + G ? hv * dk : (H + G) * dk + (hv - H - G) * dv);
+    if (!isq && !store) continue;
+    float f = isq ? temp : 1.f;
+    if (isq || isk ? qk_unit : v_unit) {
+      float ss = 0.f;
+      for (int i = lane; i < n; i += 64) ss += src[i] * src[i];
+      ss = wave_sum(ss);
+      f /= sqrtf(ss / (float)n + eps);
+    }
+    T* dst = isq ? q_out + (t * H + hv) * dk
+                 : isk ? k_cache + ((blk * G + (hv - H)) * bs + off) * dk
+                       : v_cache + ((blk * G + (hv - H - G)) * bs + off) * dv;
+    for (int i = lane; i < n; i += 64) dst[i] = from_f<T>(src[i] * f);
+  }
+}
+
 constexpr int MAX_DV_PER_LANE = 16;    // dv <= 1024
 
 // scaled score -> cap * tanh(score / cap) when a cap is set
@@ -699,6 +737,16 @@ void launch_rope_kv_store(int dtype, const void* qkv, int64_t qkv_stride,
   KGC_DISPATCH_T(dtype, rope_kv_store_kernel<T><<<T_, 256, 0, s>>>(
       (const T*)qkv, qkv_stride, positions, table, rot, table_rows, (T*)q_out, (T*)k_cache,
       (T*)v_cache, slots, H, G, dk, dv, bs, num_blocks, interleaved));
+}
+
+void launch_norm_kv_store(int out_dtype, const float* qkv, int64_t qs, const int64_t* positions,
+                          void* q_out, void* k_cache, void* v_cache, const int64_t* slots, int T_,
+                          int H, int G, int dk, int dv, int bs, int num_blocks, float eps,
+                          bool qk_unit, bool v_unit, float coef, int every, hipStream_t s) {
+  if (T_ <= 0) return;
+  KGC_DISPATCH_T(out_dtype, norm_kv_store_kernel<T><<<T_, 256, 0, s>>>(
+      qkv, qs, positions, (T*)q_out, (T*)k_cache, (T*)v_cache, slots, H, G, dk, dv, bs,
+      num_blocks, eps, qk_unit, v_unit, coef, every));
 }
 
 int window_attention_max_dv() { return 64 * MAX_DV_PER_LANE; }

@@ -354,11 +354,11 @@ void launch_moe_finish(int dtype, void* out, const void* routed, const void* den
 // `dtype`: activation type of the projection columns read (x / dt / ba / gate) and of the
 // gated norm's output; convolution and scan outputs are fp32
 int causal_conv_max_taps();
-void launch_causal_conv(int dtype, float* out, const void* x, int64_t xs, const float* w,
-                        const float* bias, float* state, const int* qsl, const int* seq_lens,
-                        const int* ctx_lens, const int* slots, const int* work_seq,
-                        const int* work_blk, int n_work, int blk_rows, int P, int D, int Tp,
-                        int C, int K, int num_slots, bool silu, hipStream_t s);
+void launch_causal_conv(int dtype, void* out, bool out_f32, const void* x, int64_t xs,
+                        const float* w, const float* bias, float* state, const int* qsl,
+                        const int* seq_lens, const int* ctx_lens, const int* slots,
+                        const int* work_seq, const int* work_blk, int n_work, int blk_rows, int P,
+                        int D, int Tp, int C, int K, int num_slots, bool silu, hipStream_t s);
 int matrix_scan_max_rows();
 void launch_ssd_scan(int dtype, float* out, const float* xbc, const void* dt, int64_t dts,
                      const float* a_log, const float* dt_bias, const float* dskip, float* S,
@@ -373,5 +373,34 @@ void launch_gated_delta_scan(int dtype, float* out, const float* qkv, const void
 void launch_gated_rms_norm(int dtype, void* out, int64_t os, const float* y, const void* gate,
                            int64_t gs, const float* w, int rows, int n, int groups, float eps,
                            bool gate_first, hipStream_t s);
+
+// ---- decay_scan.hip / Lorenex-style decoders ----------------------------------------------
+int decay_scan_max_rows();
+int gla_scan_max_rank();
+void launch_gla_scan(int dtype, float* out, const void* proj, int64_t ps, const void* low,
+                     int64_t ls, const float* a2, const float* a2b, float* S, const int* qsl,
+                     const int* seq_lens, const int* ctx_lens, const int* slots, int P, int D,
+                     int Tp, int H, int d, int V, int R, float tau, int num_slots,
+                     hipStream_t s);
+void launch_selective_scan(int dtype, void* out, int64_t os, const void* x, const void* dt,
+                           const void* bc, int64_t bcs, const float* At, const float* dt_bias,
+                           const float* dskip, const void* z, int64_t zs, float* S,
+                           const int* qsl, const int* seq_lens, const int* ctx_lens,
+                           const int* slots, int P, int D, int Tp, int I, int N,
+                           float out_scale, int num_slots, hipStream_t s);
+void launch_norm_kv_store(int out_dtype, const float* qkv, int64_t qs, const int64_t* positions,
+                          void* q_out, void* k_cache, void* v_cache, const int64_t* slots, int T_,
+                          int H, int G, int dk, int dv, int bs, int num_blocks, float eps,
+                          bool qk_unit, bool v_unit, float coef, int every, hipStream_t s);
+void launch_polynorm(int dtype, void* out, const void* z, const float* coef, int64_t rows, int F,
+                     float eps, hipStream_t s);
+void launch_swiglu_clamp(int dtype, void* out, const void* x, int64_t rows, int I, float limit,
+                         float alpha, hipStream_t s);
+void launch_embed_pos(int dtype, float* out, const int64_t* ids, const int64_t* positions,
+                      const void* table, const float* pos, int T_, int W, int vocab, int max_pos,
+                      float scale, hipStream_t s);
+void launch_moe_route_softmax_all(float* w, int* ids, float* idw, const float* logits,
+                                  int64_t stride, const float* corr, int ntok, int E, int k,
+                                  int n_real, hipStream_t s);
 
 }  // namespace kgc

@@ -742,4 +742,100 @@ void launch_moe_finish(int dtype, void* out, const void* routed, const void* den
                                                   (const float*)shared, gate, gs, ntok, E, k, W);
 }
 
+// ---- softmax routing over all router outputs with a choice correction ----------------------
+// One wave per token.  s = softmax(logits) over all E outputs; k rounds of a wave-wide arg-max
+// over s + correction (the lowest index wins among equals); a chosen output's weight is its s,
+// unchanged.  Outputs >= n_real are identity experts: their pairs get weight 0 and their
+// scores are summed into idw[t].
+namespace {
+
+template <int PER_LANE>                      // outputs per lane: E <= 64 * PER_LANE
+__global__ __launch_bounds__(256) void moe_route_softmax_all_kernel(
+    float* __restrict__ w, int* __restrict__ ids, float* __restrict__ idw,
+    const float* __restrict__ logits, int64_t stride, const float* __restrict__ corr, int ntok,
+    int E, int k, int n_real) {
+  const int t = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (t >= ntok) return;
+  const float* lr = logits + (int64_t)t * stride;
+  float sc[PER_LANE], ch[PER_LANE];
+  float mx = -INFINITY;
+#pragma unroll
+  for (int u = 0; u < PER_LANE; ++u) {
+    const int e = lane + 64 * u;
+    sc[u] = e < E ? lr[e] : -INFINITY;
+    mx = fmaxf(mx, sc[u]);
+  }
+  mx = wave_max(mx);
+  float sum = 0.f;
+#pragma unroll
+  for (int u = 0; u < PER_LANE; ++u) {
+    sc[u] = lane + 64 * u < E ? expf(sc[u] - mx) : 0.f;
+    sum += sc[u];
+  }
+  sum = wave_sum(sum);
+  const float inv = 1.f / sum;
+#pragma unroll
+  for (int u = 0; u < PER_LANE; ++u) {
+    const int e = lane + 64 * u;
+    sc[u] *= inv;
+    ch[u] = e < E ? sc[u] + corr[e] : -INFINITY;
+  }
+  float mine = 0.f, side = 0.f;         // lane j keeps the j-th chosen score
+  int mine_id = 0;
+  for (int j = 0; j < k; ++j) {
+    float best = -INFINITY, bs = 0.f;
+    int bi = 0x7fffffff;
+#pragma unroll
+    for (int u = 0; u < PER_LANE; ++u) {
+      if (ch[u] > best) {               // strict: the lowest index of a lane's equals
+        best = ch[u];
+        bi = lane + 64 * u;
+        bs = sc[u];
+      }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ob = __shfl_xor(best, o, 64), os = __shfl_xor(bs, o, 64);
+      const int oi = __shfl_xor(bi, o, 64);
+      if (ob > best || (ob == best && oi < bi)) {
+        best = ob;
+        bi = oi;
+        bs = os;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < PER_LANE; ++u)
+      if (lane + 64 * u == bi) ch[u] = -INFINITY;
+    const bool ident = bi >= n_real;
+    if (ident) side += bs;
+    if (j == lane) {                    // host checks k <= 64
+      mine = ident ? 0.f : bs;
+      mine_id = bi < E ? bi : 0;
+    }
+  }
+  if (lane < k) {
+    w[(int64_t)t * k + lane] = mine;
+    ids[(int64_t)t * k + lane] = mine_id;
+  }
+  if (lane == 0) idw[t] = side;
+}
+
+}  // namespace
+
+void launch_moe_route_softmax_all(float* w, int* ids, float* idw, const float* logits,
+                                  int64_t stride, const float* corr, int ntok, int E, int k,
+                                  int n_real, hipStream_t s) {
+  if (ntok <= 0) return;
+  const int grid = (ntok + 3) / 4;
+  if (E <= 64)
+    moe_route_softmax_all_kernel<1><<<grid, 256, 0, s>>>(w, ids, idw, logits, stride, corr, ntok,
+                                                         E, k, n_real);
+  else if (E <= 256)
+    moe_route_softmax_all_kernel<4><<<grid, 256, 0, s>>>(w, ids, idw, logits, stride, corr, ntok,
+                                                         E, k, n_real);
+  else
+    moe_route_softmax_all_kernel<RS_MAX_PER_LANE><<<grid, 256, 0, s>>>(
+        w, ids, idw, logits, stride, corr, ntok, E, k, n_real);
+}
+
 }  // namespace kgc

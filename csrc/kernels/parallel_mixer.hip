@@ -95,11 +95,26 @@ __device__ __forceinline__ void store_f32(float* p, const float (&v)[VEC]) {
   else *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
 }
 
+// VEC adjacent output channels in the output's type (fp32, or the 16-bit input type)
+template <typename O, int VEC>
+__device__ __forceinline__ void store_out(O* p, const float (&v)[VEC]) {
+  if constexpr (std::is_same_v<O, float>) {
+    store_f32<VEC>(p, v);
+  } else if constexpr (VEC == 1) {
+    p[0] = from_f<O>(v[0]);
+  } else {
+    Pack4<O> t;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) t.h[e] = from_f<O>(v[e]);
+    *reinterpret_cast<u32x2*>(p) = t.u;
+  }
+}
+
 // VEC: adjacent channels per thread (4 where the column slice, the channel count and the
 // row stride allow 8- / 16-byte accesses, else 1)
-template <typename T, int K, int VEC>
+template <typename T, typename O, int K, int VEC>
 __global__ __launch_bounds__(NT) void causal_conv_kernel(
-    float* __restrict__ out, const T* __restrict__ x, int64_t xs, const float* __restrict__ w,
+    O* __restrict__ out, const T* __restrict__ x, int64_t xs, const float* __restrict__ w,
     const float* __restrict__ bias, float* __restrict__ state, const int* __restrict__ qsl,
     const int* __restrict__ seq_lens, const int* __restrict__ ctx_lens,
     const int* __restrict__ slots, const int* __restrict__ work_seq,
@@ -120,12 +135,12 @@ __global__ __launch_bounds__(NT) void causal_conv_kernel(
   const int c = (blockIdx.y * NT + threadIdx.x) * VEC;
   if (c >= C || r0 >= q.len) return;
   const int nrows = min(CV_ROWS, q.len - r0);
-  float* orow = out + (int64_t)(q.start + r0) * C + c;
+  O* orow = out + (int64_t)(q.start + r0) * C + c;
   if (q.slot < 0 || q.slot >= num_slots || q.pos0 < 0) {
     float z[VEC];
 #pragma unroll
     for (int v = 0; v < VEC; ++v) z[v] = 0.f;
-    for (int r = 0; r < nrows; ++r) store_f32<VEC>(orow + (int64_t)r * C, z);
+    for (int r = 0; r < nrows; ++r) store_out<O, VEC>(orow + (int64_t)r * C, z);
     return;
   }
   const bool fresh = q.pos0 == 0;
@@ -177,7 +192,7 @@ __global__ __launch_bounds__(NT) void causal_conv_kernel(
 #pragma unroll
         for (int v = 0; v < VEC; ++v) win[K - 2][v] = in[u][v];
       }
-      if (rb + u < nrows) store_f32<VEC>(orow + (int64_t)(rb + u) * C, y);
+      if (rb + u < nrows) store_out<O, VEC>(orow + (int64_t)(rb + u) * C, y);
     }
   }
   if (r0 == 0) {
@@ -472,11 +487,11 @@ __global__ __launch_bounds__(NT) void gated_rms_norm_kernel(
 
 int causal_conv_max_taps() { return CV_KMAX; }
 
-void launch_causal_conv(int dtype, float* out, const void* x, int64_t xs, const float* w,
-                        const float* bias, float* state, const int* qsl, const int* seq_lens,
-                        const int* ctx_lens, const int* slots, const int* work_seq,
-                        const int* work_blk, int n_work, int blk_rows, int P, int D, int Tp,
-                        int C, int K, int num_slots, bool silu, hipStream_t s) {
+void launch_causal_conv(int dtype, void* out, bool out_f32, const void* x, int64_t xs,
+                        const float* w, const float* bias, float* state, const int* qsl,
+                        const int* seq_lens, const int* ctx_lens, const int* slots,
+                        const int* work_seq, const int* work_blk, int n_work, int blk_rows, int P,
+                        int D, int Tp, int C, int K, int num_slots, bool silu, hipStream_t s) {
   const int items = n_work * (blk_rows / CV_ROWS) + D;
   if (items <= 0 || C <= 0) return;
   // four channels per thread where every access is then an aligned 8- or 16-byte one
@@ -486,10 +501,12 @@ void launch_causal_conv(int dtype, float* out, const void* x, int64_t xs, const 
                    reinterpret_cast<uintptr_t>(state) % 16 == 0;
   const int per = NT * (vec ? 4 : 1);
   const dim3 grid(items, (C + per - 1) / per);
+#define KGC_CV_O(KK, V, O)                                                                   \
+  causal_conv_kernel<T, O, KK, V><<<grid, NT, 0, s>>>(                                       \
+      (O*)out, (const T*)x, xs, w, bias, state, qsl, seq_lens, ctx_lens, slots, work_seq, work_blk, \
+      n_work, blk_rows, P, Tp, C, num_slots, silu)
 #define KGC_CV_V(KK, V)                                                                      \
-  KGC_PM_DISPATCH_T(dtype, causal_conv_kernel<T, KK, V><<<grid, NT, 0, s>>>(                 \
-      out, (const T*)x, xs, w, bias, state, qsl, seq_lens, ctx_lens, slots, work_seq, work_blk, \
-      n_work, blk_rows, P, Tp, C, num_slots, silu))
+  KGC_PM_DISPATCH_T(dtype, if (out_f32) KGC_CV_O(KK, V, float); else KGC_CV_O(KK, V, T))
 #define KGC_CV(KK)                                    \
   do {                                                \
     if (vec) KGC_CV_V(KK, 4); else KGC_CV_V(KK, 1);   \
@@ -506,6 +523,7 @@ void launch_causal_conv(int dtype, float* out, const void* x, int64_t xs, const 
   }
 #undef KGC_CV
 #undef KGC_CV_V
+#undef KGC_CV_O
 }
 
 int matrix_scan_max_rows() { return 256; }

@@ -302,7 +302,7 @@ class LorenexForCausalLM(nn.Module):
         if leaf == "o":
             return put(mix.o_proj.weight.data[:, mix.left.n_out:], w)
         if leaf == "A_log":
-            return put(core.A.data, -torch.exp(w.float()))
+            return put(core.A.data, -torch.exp(w.float()).t())
         tgt = {"conv": core.conv_w, "conv.b": core.conv_b, "x": core.x_proj.weight,
                "dt": core.dt_proj.weight, "dt.b": core.dt_bias, "D": core.dskip}.get(leaf)
         return tgt is not None and put(tgt.data, w)

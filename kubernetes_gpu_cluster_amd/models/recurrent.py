@@ -216,7 +216,8 @@ class MambaCore(nn.Module):
     SiLU (the last taps - 1 inputs are per-sequence state); W_x x = dt | B | C (dt_rank, N,
     N); d = softplus(W_dt dt + dt_bias) per channel; with A = -exp(A_log) [width, N]:
         S[c, n] = exp(d_c A[c, n]) S[c, n] + d_c x_c B_n,   y_c = S[c, :] . C + D_c x_c
-    (S fp32, per-sequence state); y * silu(z) (times ``out_scale``) is written into a column
+    (S fp32, per-sequence state, kept as [N, width] like A so that loads run along the
+    channels); y * silu(z) (times ``out_scale``) is written into a column
     slice of the output projection's input.  The two inner projections are GEMMs; step
     sizes, decays and the state are fp32."""
 
@@ -230,13 +231,13 @@ class MambaCore(nn.Module):
         f = lambda *s: nn.Parameter(torch.zeros(*s, dtype=torch.float32, device=device),  # noqa: E731
                                     requires_grad=False)
         self.conv_w, self.conv_b = f(I, spec.conv), f(I)
-        self.A = f(I, N)                         # -exp(A_log)
+        self.A = f(N, I)                         # -exp(A_log), states by channels
         self.dt_bias, self.dskip = f(I), f(I)
 
     def state_shapes(self) -> tuple:
         """Per-slot shapes: the convolution's last inputs, the recurrent state."""
         sp = self.spec
-        return ((max(sp.conv - 1, 1), sp.width), (sp.width, sp.dim))
+        return ((max(sp.conv - 1, 1), sp.width), (sp.dim, sp.width))
 
     def forward(self, proj: torch.Tensor, col0: int, ctx: ForwardContext, state: tuple,
                 out: torch.Tensor) -> None:

@@ -1085,18 +1085,19 @@ def gla_scan(proj: torch.Tensor, low: torch.Tensor, a2: torch.Tensor, a2_bias: t
     return out
 
 
-def selective_scan(x: torch.Tensor, dt: torch.Tensor, bc: torch.Tensor, A: torch.Tensor,
+def selective_scan(x: torch.Tensor, dt: torch.Tensor, bc: torch.Tensor, At: torch.Tensor,
                    dt_bias: torch.Tensor, dskip: torch.Tensor, z: torch.Tensor,
                    state: torch.Tensor, meta, out_scale: float, out: torch.Tensor) -> torch.Tensor:
     """out [T, I] (a column slice of a wider buffer) = y * silu(z) * out_scale, y the
-    selective scan over every step sequence's rows from / into state [slots, I, N]; x, dt
-    [T, I], bc [T, 2 N] and z [T, I] (column slices), A fp32 [I, N]; see
+    selective scan over every step sequence's rows from / into state [slots, N, I]; x, dt
+    [T, I], bc [T, 2 N] and z [T, I] (column slices), At fp32 [N, I]; see
     ``ref.selective_scan``."""
     if not _gpu(x):
-        out.copy_(ref.selective_scan(x, dt, bc, A, dt_bias, dskip, z, state,
+        out.copy_(ref.selective_scan(x, dt, bc, At, dt_bias, dskip, z, state,
                                      ref.step_sequences(meta), out_scale, out.dtype))
         return out
-    _k().selective_scan(out, x, dt, bc, A, dt_bias, dskip, z, state, meta.query_start_loc,
+    _k().selective_scan(out, x, dt.contiguous(), bc, At, dt_bias, dskip, z, state,
+                        meta.query_start_loc,
                         meta.prefill_seq_lens, meta.decode_ctx_lens, meta.state_slots,
                         meta.num_prefills, meta.num_decodes, meta.num_prefill_tokens,
                         float(out_scale))

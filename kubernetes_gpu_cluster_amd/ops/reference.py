@@ -868,18 +868,18 @@ def gla_scan(proj: torch.Tensor, low: torch.Tensor, a2: torch.Tensor, a2_bias: t
     return out.view(T, H * dv)
 
 
-def selective_scan(x: torch.Tensor, dt: torch.Tensor, bc: torch.Tensor, A: torch.Tensor,
+def selective_scan(x: torch.Tensor, dt: torch.Tensor, bc: torch.Tensor, At: torch.Tensor,
                    dt_bias: torch.Tensor, dskip: torch.Tensor, z: torch.Tensor,
                    state: torch.Tensor, seqs: list, out_scale: float,
                    out_dtype: torch.dtype) -> torch.Tensor:
     """The selective scan.  x [T, I] (after convolution and SiLU), dt [T, I] raw step sizes,
-    bc [T, 2 N] = B | C, A fp32 [I, N] (negative), z [T, I] the gate pre-activation.  With
-    d = softplus(dt + dt_bias), per channel c and state n:
-        S[c, n] = exp(d_c A[c, n]) S[c, n] + d_c x_c B_n;   y_c = sum_n S[c, n] C_n + dskip_c x_c
-    from state[slot] [I, N] fp32 (zeros at position 0), written back.
+    bc [T, 2 N] = B | C, At fp32 [N, I] (negative; states by channels), z [T, I] the gate
+    pre-activation.  With d = softplus(dt + dt_bias), per channel c and state n:
+        S[n, c] = exp(d_c At[n, c]) S[n, c] + d_c x_c B_n;   y_c = sum_n S[n, c] C_n + dskip_c x_c
+    from state[slot] [N, I] fp32 (zeros at position 0), written back.
     -> y * silu(z) * out_scale in out_dtype [T, I]."""
     T, I = x.shape
-    N = A.shape[1]
+    N = At.shape[0]
     xf = x.float()
     d = torch.nn.functional.softplus(dt.float() + dt_bias.float())
     B, C = bc[:, :N].float(), bc[:, N: 2 * N].float()
@@ -887,10 +887,10 @@ def selective_scan(x: torch.Tensor, dt: torch.Tensor, bc: torch.Tensor, A: torch
     for a, n, p0, slot in seqs:
         if slot < 0:
             continue
-        S = torch.zeros(I, N) if p0 == 0 else state[slot].clone()
+        S = torch.zeros(N, I) if p0 == 0 else state[slot].clone()
         for t in range(a, a + n):
-            S = torch.exp(d[t][:, None] * A.float()) * S + (d[t] * xf[t])[:, None] * B[t][None, :]
-            y[t] = S @ C[t] + dskip.float() * xf[t]
+            S = torch.exp(d[t][None, :] * At.float()) * S + B[t][:, None] * (d[t] * xf[t])[None, :]
+            y[t] = C[t] @ S + dskip.float() * xf[t]
         state[slot] = S
     zf = z.float()
     return (y * (zf * torch.sigmoid(zf)) * out_scale).to(out_dtype)
