@@ -780,10 +780,18 @@ def lorenex_config(d: dict, name: str, shapes: Optional[dict] = None) -> ModelCo
     tensor name -> shape of the checkpoint beside it, for the sizes config.json leaves to
     the tensors."""
     layers = d["layers"]
-    share = tuple(int(e.get("weights_of", i)) for i, e in enumerate(layers))
-    for i, j in enumerate(share):
-        if not 0 <= j < len(layers) or share[j] != j or layers[j]["type"] != layers[i]["type"]:
-            raise ValueError(f"layer {i}: bad weights_of {j}")
+    share = []
+    for i, e in enumerate(layers):
+        j, seen = i, set()
+        while "weights_of" in layers[j] and int(layers[j]["weights_of"]) != j:
+            seen.add(j)                     # a layer may point at one that points further
+            j = int(layers[j]["weights_of"])
+            if not 0 <= j < len(layers) or j in seen:
+                raise ValueError(f"layer {i}: bad weights_of")
+        if layers[j]["type"] != e["type"]:
+            raise ValueError(f"layer {i} runs with the weights of layer {j}, of another type")
+        share.append(j)
+    share = tuple(share)
     specs = []
     for i, e in enumerate(layers):
         a1 = (shapes or {}).get(f"l{share[i]}.mix.a1")

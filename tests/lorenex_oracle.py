@@ -141,12 +141,19 @@ def polynorm_mlp(h, W, p, eps):
     return (a * rms(z, eps) + b * rms(z ** 2, eps) + c * rms(z ** 3, eps) + e) @ W[p + "down"].T
 
 
-def route(h, W, p, top):
-    """-> (weights [T, top], expert ids [T, top]); ids >= experts name identity experts."""
+def route(h, W, p, top, margins=None):
+    """-> (weights [T, top], expert ids [T, top]); ids >= experts name identity experts.
+    ``margins`` receives, per token, how far the last chosen output's choice score lies above
+    the first one left out, relative to the chosen scores' size."""
     z = h @ W[p + "router"].T
     s = np.exp(z - z.max(-1, keepdims=True))
     s = s / s.sum(-1, keepdims=True)
-    ids = np.argsort(-(s + W[p + "correction"]), axis=-1, kind="stable")[:, :top]
+    c = s + W[p + "correction"]
+    order = np.argsort(-c, axis=-1, kind="stable")
+    ids = order[:, :top]
+    if margins is not None and top < c.shape[1]:
+        cs = np.take_along_axis(c, order, 1)
+        margins.append((cs[:, top - 1] - cs[:, top]) / np.abs(cs[:, :top]).max(-1))
     return np.take_along_axis(s, ids, 1), ids
 
 
@@ -156,9 +163,9 @@ def expert(h, W, p, limit):
     return (g * sigmoid(1.702 * g) * (u + 1.0)) @ W[p + "down"].T
 
 
-def moe_mlp(h, W, p, mlp):
+def moe_mlp(h, W, p, mlp, margins=None):
     E, top, limit = mlp["router"]["experts"], mlp["router"]["top"], mlp["expert"]["limit"]
-    w, ids = route(h, W, p, top)
+    w, ids = route(h, W, p, top, margins)
     out = np.zeros_like(h)
     for t in range(h.shape[0]):
         for j in range(top):
@@ -169,14 +176,18 @@ def moe_mlp(h, W, p, mlp):
 
 
 # ------------------------------------------------------------------ the model
-def forward(cfg: dict, W: dict, tokens, taps: list = None):
-    """-> logits [T, vocab]; ``taps`` receives the residual stream after every layer."""
+def forward(cfg: dict, W: dict, tokens, taps: list = None, margins: list = None):
+    """-> logits [T, vocab]; ``taps`` receives the residual stream after every layer,
+    ``margins`` every routed layer's routing margins (see ``route``)."""
     eps, m = cfg["norm"]["eps"], cfg.get("residual_mult", 1.0)
     tokens = np.asarray(tokens)
     T = len(tokens)
     x = W["embed"][tokens] * cfg.get("embedding", {}).get("scale", 1.0) + W["pos"][:T]
     for i, L in enumerate(cfg["layers"]):
-        p = f"l{L.get('weights_of', i)}."
+        j = i
+        while cfg["layers"][j].get("weights_of", j) != j:
+            j = cfg["layers"][j]["weights_of"]
+        p = f"l{j}."
         if L["type"] == "gla":
             y = gla_mixer(x, W, p + "mix.", L["mixer"], eps)
         elif L["type"] == "parallel":
@@ -187,7 +198,7 @@ def forward(cfg: dict, W: dict, tokens, taps: list = None):
         mlp = L.get("mlp")
         if mlp:
             y = (polynorm_mlp(x, W, p + "mlp.", eps) if mlp["kind"] == "dense"
-                 else moe_mlp(x, W, p + "mlp.", mlp))
+                 else moe_mlp(x, W, p + "mlp.", mlp, margins))
             x = x + m * rms(y, eps) * W[p + "norm2"]
         if taps is not None:
             taps.append(x.copy())
