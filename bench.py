@@ -91,8 +91,8 @@ def parse():
     ap.add_argument("--compare-sizes", default="w2048,w4096",
                     help="--mode compare: size suffixes of the <family>-<size> presets")
     ap.add_argument("--compare-families", default="dilavik,llama",
-                    help="--mode compare: the preset families to run at each size (nolesun, dilavik, "
-                         "konovik, llama); ratios are taken against the last one")
+                    help="--mode compare: the preset families to run at each size (lorenex, nolesun, "
+                         "dilavik, konovik, llama); ratios are taken against the last one")
     ap.add_argument("--mode", default="service", choices=["service", "engine", "compare"],
                     help="service: HTTP/SSE through API server + router (headline); "
                          "engine: LLMEngine.step() in-process")
@@ -643,7 +643,7 @@ def _compare_one(model: str, args) -> dict:
 
 
 def main_compare(args):
-    """--mode compare: the hybrid presets (nolesun, dilavik, konovik) beside the Llama-style decoders of equal size
+    """--mode compare: the hybrid presets (lorenex, nolesun, dilavik, konovik) beside the Llama-style decoders of equal size
     (models/configs.py), same requests, same engine settings, one JSON line per model and a
     closing line with the ratios.  Random weights, synthetic prompts."""
     assert torch.cuda.is_available(), "bench.py --mode compare needs a GPU"

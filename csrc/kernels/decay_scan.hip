@@ -15,10 +15,12 @@
 // S [R, V] (gla: R key channels, V value columns; selective scan: R states, V channels, kept
 // in memory as [states, channels] so that a wave's loads are contiguous).  A wave owns 16
 // columns (4 when few long sequences have to cover the chip); its lanes are (row group
-// rg = lane / columns, column) and a lane keeps rows rg, rg + NRG, ... of its column in
-// registers for the whole chunk: S is read and written once per step, and a token's sum over
-// rows ends with cross-lane steps inside the wave -- no barrier per token.  Tokens are
-// staged in LDS 16 at a time.
+// rg = lane / columns, column) and a lane keeps the RPT consecutive rows rg RPT .. of its
+// column in registers for the whole chunk: S is read and written once per step, a token's
+// per-row vectors come from LDS four rows per 16-byte read (a row group's rows lie together,
+// groups 16 bytes apart in banks), and a token's sum over rows ends with cross-lane steps
+// inside the wave -- no barrier per token.  Tokens are staged in LDS 16 at a time (only the
+// tokens present: a decode row stages one).
 #include "common.h"
 #include "launch.h"
 
@@ -59,6 +61,13 @@ __device__ __forceinline__ float logsigmoid_f(float x) {
   return fminf(x, 0.f) - log1pf(expf(-fabsf(x)));
 }
 
+// LDS place of state row r when a lane owns RPT consecutive rows: row groups are padded by
+// four floats so that the groups' 16-byte reads fall into different banks
+template <int RPT>
+__device__ __forceinline__ int lrow(int r) { return r + 4 * (r / RPT); }
+
+__device__ __forceinline__ float4 lds4(const float* p) { return *reinterpret_cast<const float4*>(p); }
+
 // ---- gated linear attention -----------------------------------------------------------------
 // proj [T, >= 2 H d + H V] (row stride ps) = q | k | v; low [T, R] (row stride ls) the decay
 // bottleneck; a2 fp32 [H d, R], a2b fp32 [H d].
@@ -72,13 +81,14 @@ __global__ __launch_bounds__(NT) void gla_scan_kernel(
     int V, int R, float inv_tau, int num_slots) {
   constexpr int CW = 1 << LOGC, NRG = 64 >> LOGC;     // columns per wave, row groups per wave
   constexpr int RP = NRG * RPT, CT = CW * (NT / 64);  // rows (padded), columns per workgroup
+  constexpr int RPS = RP + 4 * NRG;                   // LDS floats per token and vector
   constexpr int NG = NT / RP > 0 ? NT / RP : 1;       // token groups of the decay projection
   constexpr int PER = (TB + NG - 1) / NG;             // ... and tokens per thread in it
   extern __shared__ float lds[];
-  float* ks = lds;                   // [TB][RP]
-  float* qs = ks + TB * RP;          // [TB][RP]
-  float* al = qs + TB * RP;          // [TB][RP] decays
-  float* vs = al + TB * RP;          // [TB][CT]
+  float* ks = lds;                   // [TB][RPS]
+  float* qs = ks + TB * RPS;         // [TB][RPS]
+  float* al = qs + TB * RPS;         // [TB][RPS] decays
+  float* vs = al + TB * RPS;         // [TB][CT]
   float* lw = vs + TB * CT;          // [TB][R]
   const int s = blockIdx.x, h = blockIdx.y;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, rg = lane >> LOGC;
@@ -97,79 +107,75 @@ __global__ __launch_bounds__(NT) void gla_scan_kernel(
   float Sr[RPT];
 #pragma unroll
   for (int i = 0; i < RPT; ++i) {
-    const int r = NRG * i + rg;
+    const int r = rg * RPT + i;
     Sr[i] = (!fresh && r < d && colok) ? Sp[(int64_t)r * V + col] : 0.f;
   }
   const float qscale = 1.f / sqrtf((float)d);
   for (int t0 = 0; t0 < q.len; t0 += TB) {
     const int nb = min(TB, q.len - t0);
-    for (int e = threadIdx.x; e < TB * RP; e += NT) {
+    for (int e = threadIdx.x; e < nb * RP; e += NT) {
       const int tb = e / RP, r = e - tb * RP;
       float kv = 0.f, qv = 0.f;
-      if (tb < nb && r < d) {
+      if (r < d) {
         const T* row = proj + (int64_t)(q.start + t0 + tb) * ps;
         kv = to_f(row[koff + r]);
         qv = to_f(row[qoff + r]) * qscale;
       }
-      ks[e] = kv;
-      qs[e] = qv;
+      ks[tb * RPS + lrow<RPT>(r)] = kv;
+      qs[tb * RPS + lrow<RPT>(r)] = qv;
     }
-    for (int e = threadIdx.x; e < TB * CT; e += NT) {
+    for (int e = threadIdx.x; e < nb * CT; e += NT) {
       const int tb = e / CT, c = blockIdx.z * CT + (e - tb * CT);
-      vs[e] = (tb < nb && c < V) ? to_f(proj[(int64_t)(q.start + t0 + tb) * ps + voff + c]) : 0.f;
+      vs[e] = c < V ? to_f(proj[(int64_t)(q.start + t0 + tb) * ps + voff + c]) : 0.f;
     }
-    for (int e = threadIdx.x; e < TB * R; e += NT) {
+    for (int e = threadIdx.x; e < nb * R; e += NT) {
       const int tb = e / R, j = e - tb * R;
-      lw[e] = tb < nb ? to_f(low[(int64_t)(q.start + t0 + tb) * ls + j]) : 0.f;
+      lw[e] = to_f(low[(int64_t)(q.start + t0 + tb) * ls + j]);
     }
     __syncthreads();
-    // decays: thread (row r, token group g) keeps its row of a2 in flight once per block
-    for (int r = threadIdx.x % RP; r < RP; r += NT) {
-      const int g0 = threadIdx.x / RP;
-      float acc[PER];
+    // decays: thread (row r, token group g0) reads its row of a2 once per block of tokens
+    {
+      const int r = threadIdx.x % RP, g0 = threadIdx.x / RP;
+      if (g0 < NG && g0 < nb) {
+        float acc[PER];
 #pragma unroll
-      for (int i = 0; i < PER; ++i) acc[i] = 0.f;
-      if (r < d) {
-        const float* ar = a2 + (int64_t)(h * d + r) * R;
-        for (int j = 0; j < R; ++j) {
-          const float a = ar[j];
+        for (int i = 0; i < PER; ++i) acc[i] = 0.f;
+        if (r < d) {
+          const float* ar = a2 + (int64_t)(h * d + r) * R;
+          for (int j = 0; j < R; ++j) {
+            const float a = ar[j];
 #pragma unroll
-          for (int i = 0; i < PER; ++i) {
-            const int tb = g0 + i * NG;
-            if (tb < TB) acc[i] += a * lw[tb * R + j];
+            for (int i = 0; i < PER; ++i) {
+              const int tb = g0 + i * NG;
+              if (tb < nb) acc[i] += a * lw[tb * R + j];
+            }
           }
         }
-        const float b = a2b[h * d + r];
+        const float b = r < d ? a2b[h * d + r] : 0.f;
 #pragma unroll
         for (int i = 0; i < PER; ++i) {
           const int tb = g0 + i * NG;
-          if (tb < TB) al[tb * RP + r] = expf(logsigmoid_f(acc[i] + b) * inv_tau);
-        }
-      } else {
-#pragma unroll
-        for (int i = 0; i < PER; ++i) {
-          const int tb = g0 + i * NG;
-          if (tb < TB) al[tb * RP + r] = 0.f;
+          if (tb < nb)
+            al[tb * RPS + lrow<RPT>(r)] = r < d ? expf(logsigmoid_f(acc[i] + b) * inv_tau) : 0.f;
         }
       }
     }
     __syncthreads();
     for (int tb = 0; tb < nb; ++tb) {
       const float vv = vs[tb * CT + lc];
-      const float* kp = ks + tb * RP + rg;
-      const float* qp = qs + tb * RP + rg;
-      const float* ap = al + tb * RP + rg;
+      const int base = tb * RPS + rg * (RPT + 4);
       float a0 = 0.f, a1 = 0.f, a2s = 0.f, a3 = 0.f;       // independent chains
 #pragma unroll
       for (int i = 0; i < RPT; i += 4) {
-        Sr[i] = ap[NRG * i] * Sr[i] + kp[NRG * i] * vv;
-        Sr[i + 1] = ap[NRG * (i + 1)] * Sr[i + 1] + kp[NRG * (i + 1)] * vv;
-        Sr[i + 2] = ap[NRG * (i + 2)] * Sr[i + 2] + kp[NRG * (i + 2)] * vv;
-        Sr[i + 3] = ap[NRG * (i + 3)] * Sr[i + 3] + kp[NRG * (i + 3)] * vv;
-        a0 += Sr[i] * qp[NRG * i];
-        a1 += Sr[i + 1] * qp[NRG * (i + 1)];
-        a2s += Sr[i + 2] * qp[NRG * (i + 2)];
-        a3 += Sr[i + 3] * qp[NRG * (i + 3)];
+        const float4 av = lds4(al + base + i), kv = lds4(ks + base + i), qv = lds4(qs + base + i);
+        Sr[i] = av.x * Sr[i] + kv.x * vv;
+        Sr[i + 1] = av.y * Sr[i + 1] + kv.y * vv;
+        Sr[i + 2] = av.z * Sr[i + 2] + kv.z * vv;
+        Sr[i + 3] = av.w * Sr[i + 3] + kv.w * vv;
+        a0 += Sr[i] * qv.x;
+        a1 += Sr[i + 1] * qv.y;
+        a2s += Sr[i + 2] * qv.z;
+        a3 += Sr[i + 3] * qv.w;
       }
       float y = (a0 + a1) + (a2s + a3);
 #pragma unroll
@@ -180,7 +186,7 @@ __global__ __launch_bounds__(NT) void gla_scan_kernel(
   }
 #pragma unroll
   for (int i = 0; i < RPT; ++i) {
-    const int r = NRG * i + rg;
+    const int r = rg * RPT + i;
     if (r < d && colok) Sp[(int64_t)r * V + col] = Sr[i];
   }
 }
@@ -199,11 +205,13 @@ __global__ __launch_bounds__(NT) void selective_scan_kernel(
     const int* __restrict__ slots, int P, int Tp, int I, int N, float out_scale, int num_slots) {
   constexpr int CW = 1 << LOGC, NRG = 64 >> LOGC;
   constexpr int RP = NRG * RPT, CT = CW * (NT / 64);
+  constexpr int RPS = RP + 4 * NRG;
   extern __shared__ float lds[];
-  float* Bs = lds;                   // [TB][RP]
-  float* Cs = Bs + TB * RP;          // [TB][RP]
-  float* xv = Cs + TB * RP;          // [TB][CT]
+  float* Bs = lds;                   // [TB][RPS]
+  float* Cs = Bs + TB * RPS;         // [TB][RPS]
+  float* xv = Cs + TB * RPS;         // [TB][CT]
   float* dv = xv + TB * CT;          // [TB][CT] step sizes
+  float* gz = dv + TB * CT;          // [TB][CT] silu(z) * out_scale
   const int s = blockIdx.x;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, rg = lane >> LOGC;
   const int lc = wave * CW + (lane & (CW - 1)), col = blockIdx.z * CT + lc;
@@ -216,70 +224,72 @@ __global__ __launch_bounds__(NT) void selective_scan_kernel(
   }
   float* Sp = S + (int64_t)q.slot * N * I;
   const bool fresh = q.pos0 == 0;
+  // Ar: A times log2(e), so that exp(d A) is one v_exp_f32 of d * Ar (d A <= 0: no overflow,
+  // and a result below the normal range is a decay of zero either way)
   float Sr[RPT], Ar[RPT];
 #pragma unroll
   for (int i = 0; i < RPT; ++i) {
-    const int r = NRG * i + rg;
+    const int r = rg * RPT + i;
     const bool ok = r < N && colok;
     Sr[i] = (!fresh && ok) ? Sp[(int64_t)r * I + col] : 0.f;
-    Ar[i] = ok ? At[(int64_t)r * I + col] : 0.f;
+    Ar[i] = ok ? At[(int64_t)r * I + col] * 1.4426950408889634f : 0.f;
   }
   const float Dc = colok ? dskip[col] : 0.f;
   for (int t0 = 0; t0 < q.len; t0 += TB) {
     const int nb = min(TB, q.len - t0);
-    for (int e = threadIdx.x; e < TB * RP; e += NT) {
+    for (int e = threadIdx.x; e < nb * RP; e += NT) {
       const int tb = e / RP, r = e - tb * RP;
       float bv = 0.f, cv = 0.f;
-      if (tb < nb && r < N) {
+      if (r < N) {
         const T* row = bc + (int64_t)(q.start + t0 + tb) * bcs;
         bv = to_f(row[r]);
         cv = to_f(row[N + r]);
       }
-      Bs[e] = bv;
-      Cs[e] = cv;
+      Bs[tb * RPS + lrow<RPT>(r)] = bv;
+      Cs[tb * RPS + lrow<RPT>(r)] = cv;
     }
-    for (int e = threadIdx.x; e < TB * CT; e += NT) {
+    for (int e = threadIdx.x; e < nb * CT; e += NT) {
       const int tb = e / CT, c = blockIdx.z * CT + (e - tb * CT);
-      float xx = 0.f, dd = 0.f;
-      if (tb < nb && c < I) {
-        const int64_t at = (int64_t)(q.start + t0 + tb) * I + c;
-        xx = to_f(x[at]);
-        dd = softplus_f(to_f(dt[at]) + dt_bias[c]);
+      float xx = 0.f, dd = 0.f, gg = 0.f;
+      if (c < I) {
+        const int64_t t = q.start + t0 + tb;
+        xx = to_f(x[t * I + c]);
+        dd = softplus_f(to_f(dt[t * I + c]) + dt_bias[c]);
+        const float zv = to_f(z[t * zs + c]);
+        gg = zv * sigmoid_f(zv) * out_scale;
       }
       xv[e] = xx;
       dv[e] = dd;
+      gz[e] = gg;
     }
     __syncthreads();
     for (int tb = 0; tb < nb; ++tb) {
       const float xc = xv[tb * CT + lc], d = dv[tb * CT + lc], xd = d * xc;
-      const float* bp = Bs + tb * RP + rg;
-      const float* cp = Cs + tb * RP + rg;
+      const int base = tb * RPS + rg * (RPT + 4);
       float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
 #pragma unroll
       for (int i = 0; i < RPT; i += 4) {
-        Sr[i] = expf(d * Ar[i]) * Sr[i] + bp[NRG * i] * xd;
-        Sr[i + 1] = expf(d * Ar[i + 1]) * Sr[i + 1] + bp[NRG * (i + 1)] * xd;
-        Sr[i + 2] = expf(d * Ar[i + 2]) * Sr[i + 2] + bp[NRG * (i + 2)] * xd;
-        Sr[i + 3] = expf(d * Ar[i + 3]) * Sr[i + 3] + bp[NRG * (i + 3)] * xd;
-        a0 += Sr[i] * cp[NRG * i];
-        a1 += Sr[i + 1] * cp[NRG * (i + 1)];
-        a2 += Sr[i + 2] * cp[NRG * (i + 2)];
-        a3 += Sr[i + 3] * cp[NRG * (i + 3)];
+        const float4 bv = lds4(Bs + base + i), cv = lds4(Cs + base + i);
+        Sr[i] = __builtin_amdgcn_exp2f(d * Ar[i]) * Sr[i] + bv.x * xd;
+        Sr[i + 1] = __builtin_amdgcn_exp2f(d * Ar[i + 1]) * Sr[i + 1] + bv.y * xd;
+        Sr[i + 2] = __builtin_amdgcn_exp2f(d * Ar[i + 2]) * Sr[i + 2] + bv.z * xd;
+        Sr[i + 3] = __builtin_amdgcn_exp2f(d * Ar[i + 3]) * Sr[i + 3] + bv.w * xd;
+        a0 += Sr[i] * cv.x;
+        a1 += Sr[i + 1] * cv.y;
+        a2 += Sr[i + 2] * cv.z;
+        a3 += Sr[i + 3] * cv.w;
       }
       float y = (a0 + a1) + (a2 + a3);
 #pragma unroll
       for (int o = CW; o < 64; o <<= 1) y += __shfl_xor(y, o, 64);
-      if (rg == 0 && colok) {
-        const int64_t t = q.start + t0 + tb;
-        const float zv = to_f(z[t * zs + col]);
-        out[t * os + col] = from_f<T>((y + Dc * xc) * (zv * sigmoid_f(zv)) * out_scale);
-      }
+      if (rg == 0 && colok)
+        out[(int64_t)(q.start + t0 + tb) * os + col] = from_f<T>((y + Dc * xc) * gz[tb * CT + lc]);
     }
     __syncthreads();
   }
 #pragma unroll
   for (int i = 0; i < RPT; ++i) {
-    const int r = NRG * i + rg;
+    const int r = rg * RPT + i;
     if (r < N && colok) Sp[(int64_t)r * I + col] = Sr[i];
   }
 }
@@ -315,10 +325,15 @@ void launch_gla_scan(int dtype, float* out, const void* proj, int64_t ps, const 
                      int Tp, int H, int d, int V, int R, float tau, int num_slots,
                      hipStream_t s) {
   if (P + D <= 0) return;
-  const bool narrow = scan_narrow(P + D, H, V);
+  bool narrow = scan_narrow(P + D, H, V);
+  // the narrow form pads 16 row groups; it has to fit 64 KB of LDS with the decay bottleneck
+  if (narrow && sizeof(float) * (size_t)(3 * TB * (pow2_at_least(d, 64) + 64) + TB * 16 + TB * R) >
+                    (size_t)64 * 1024)
+    narrow = false;
   const int ct = narrow ? 16 : 64, rp = pow2_at_least(d, narrow ? 64 : 16);
+  const int rps = rp + 4 * (narrow ? 16 : 4);
   const dim3 grid(P + D, H, (V + ct - 1) / ct);
-  const size_t lds = sizeof(float) * (size_t)(3 * TB * rp + TB * ct + TB * R);
+  const size_t lds = sizeof(float) * (size_t)(3 * TB * rps + TB * ct + TB * R);
 #define KGC_GLA_W(RR, L)                                                                     \
   KGC_DS_DISPATCH_T(dtype, gla_scan_kernel<T, RR, L><<<grid, NT, lds, s>>>(                  \
       out, (const T*)proj, ps, (const T*)low, ls, a2, a2b, S, qsl, seq_lens, ctx_lens, slots, P, \
@@ -346,8 +361,9 @@ void launch_selective_scan(int dtype, void* out, int64_t os, const void* x, cons
   if (P + D <= 0) return;
   const bool narrow = scan_narrow(P + D, 1, I);
   const int ct = narrow ? 16 : 64, rp = pow2_at_least(N, narrow ? 64 : 16);
+  const int rps = rp + 4 * (narrow ? 16 : 4);
   const dim3 grid(P + D, 1, (I + ct - 1) / ct);
-  const size_t lds = sizeof(float) * (size_t)(2 * TB * rp + 2 * TB * ct);
+  const size_t lds = sizeof(float) * (size_t)(2 * TB * rps + 3 * TB * ct);
 #define KGC_SEL_W(RR, L)                                                                     \
   KGC_DS_DISPATCH_T(dtype, selective_scan_kernel<T, RR, L><<<grid, NT, lds, s>>>(            \
       (T*)out, os, (const T*)x, (const T*)dt, (const T*)bc, bcs, At, dt_bias, dskip,          \

@@ -79,15 +79,16 @@ MIXED = config([glal(gla(), dense()), par(att(), ssm(), moe()),
                 glal(gla(heads=3, dim=8, vdim=16, tau=16.0, rank=2), moe(top=3, identity=2))])
 # values a model may make equal or 1, and parts it may leave out: one head, one state, one
 # expert used of two, no identity expert, no feed-forward, a convolution of one tap and of two,
-# scales and the residual multiplier 1, value size = key size, a layer that runs with the
-# weights of one that itself names another, the parallel layer first
-PLAIN = config([par(att(heads=1, kv=1, dim=16, vdim=16, conv=1, scale=1.0, coef=1.0, every=1),
+# scales and the residual multiplier 1, a query factor that steps at every position, value
+# size = key size, a layer that runs with the weights of one that itself names another, the
+# parallel layer first
+PLAIN = config([par(att(heads=1, kv=1, dim=16, vdim=16, conv=1, scale=1.0, coef=0.25, every=1),
                     ssm(inner=16, state=1, dt_rank=1, conv=1), dense(32), ls=1.0, rs=1.0),
                 glal(gla(heads=1, dim=16, vdim=16, tau=1.0, rank=1), moe(experts=2, top=1, ff=16, identity=0)),
-                par(att(heads=1, kv=1, dim=16, vdim=16, conv=1, scale=1.0, coef=1.0, every=1),
+                par(att(heads=1, kv=1, dim=16, vdim=16, conv=1, scale=1.0, coef=0.25, every=1),
                     ssm(inner=16, state=1, dt_rank=1, conv=1), dense(32), ls=1.0, rs=1.0, weights_of=0),
                 glal(gla(heads=2, dim=8, vdim=8, tau=2.0, rank=3)),
-                par(att(heads=1, kv=1, dim=16, vdim=16, conv=1, scale=1.0, coef=1.0, every=1),
+                par(att(heads=1, kv=1, dim=16, vdim=16, conv=1, scale=1.0, coef=0.25, every=1),
                     ssm(inner=16, state=1, dt_rank=1, conv=1), dense(32), ls=1.0, rs=1.0, weights_of=2),
                 par(att(heads=2, kv=2, dim=8, vdim=8, conv=2, scale=0.7, coef=0.0, every=3),
                     ssm(inner=8, state=4, dt_rank=2, conv=2))],

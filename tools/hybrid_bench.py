@@ -1,6 +1,7 @@
 """Microbenchmarks of the hybrid-decoder kernels beside the Llama-path kernel each one is
 closest to, at the layer shapes of the dilavik-w2048 / konovik-w2048 / nolesun-w2048 /
-llama-w2048 presets (``--only nolesun``: the parallel mixers' kernels).
+llama-w2048 presets (``--only nolesun``: the parallel mixers' kernels; ``--only lorenex``: gated
+linear attention, the selective scan, unit-RMS attention inputs, PolyNorm, clamped experts).
 
     python tools/hybrid_bench.py [--reps 20] > profiles/hybrid_kernels.jsonl
 
@@ -360,6 +361,93 @@ def nolesun(reps):
                  tflop=keys * H * 4 * d / 1e12 if P_q else None, like="window_attention")
 
 
+def lorenex(reps):
+    """The Lorenex kernels at the lorenex-w2048 layer shapes, each beside the closest kernel of
+    the other decoders at the same shape (``like``)."""
+    W = 2048
+    shapes = (("prefill 32x512", [512] * 32, []), ("prefill 2x8192", [8192] * 2, []),
+              ("decode 64", [], [544] * 64), ("decode 256", [], [544] * 256))
+    for name, P_q, D_ctx in shapes:
+        n = len(P_q) + len(D_ctx)
+        m, _, nb = meta(P_q, list(P_q), D_ctx, 32, DEV, slots=list(range(n)))
+        T = sum(P_q) + len(D_ctx)
+        pos = torch.arange(T, dtype=torch.int64, device=DEV) % 512
+        slots = torch.arange(T, dtype=torch.int64, device=DEV) + 32
+        # gated linear attention: 8 heads of 128 x 256, decay bottleneck 16
+        H, d, V, R = 8, 128, 256, 16
+        proj = torch.randn(T, 2 * H * d + 2 * H * V + R, device=DEV, dtype=BF)
+        a2, a2b = torch.randn(H * d, R, device=DEV) * 0.3, torch.randn(H * d, device=DEV) + 3
+        S = torch.zeros(n, H, d, V, device=DEV)
+        us = timed(lambda: ops.gla_scan(proj, proj[:, -R:], a2, a2b, S, m, H, d, V, 16.0), reps)
+        emit("gla_scan", name, us, gbytes=2 * n * H * d * V * 4 / 1e9,
+             tflop=4 * T * H * d * V / 1e12, like="gated_delta_scan")
+        S2 = torch.zeros(n, 16, 128, 128, device=DEV)
+        qkv = torch.randn(T, 2 * 8 * 128 + 16 * 128, device=DEV)
+        par = (torch.rand(16, device=DEV), torch.randn(16, device=DEV) - 2)
+        us = timed(lambda: ops.gated_delta_scan(qkv, proj[:, :32], *par, S2, m, 16, 8, 128, 128), reps)
+        emit("gated_delta_scan (same state bytes)", name, us, gbytes=2 * n * 16 * 128 * 128 * 4 / 1e9,
+             tflop=6 * T * 16 * 128 * 128 / 1e12)
+        # attention inputs: 16 query / 4 key-value heads of 128, 4 taps, unit-RMS vectors
+        Hq, G, dk, K = 16, 4, 128, 4
+        C = (Hq + 2 * G) * dk
+        aproj = torch.randn(T, C + 2 * W, device=DEV, dtype=BF)
+        cw = torch.randn(C, K, device=DEV) * 0.3
+        cst = torch.zeros(n, K - 1, C, device=DEV)
+        us = timed(lambda: ops.causal_conv(aproj[:, :C], cw, None, cst, m, False), reps)
+        emit("causal_conv (q | k | v, 4 taps, no activation)", name, us, gbytes=T * C * 6 / 1e9,
+             like="causal_conv")
+        conv = torch.randn(T, C, device=DEV)
+        kc = torch.zeros(nb + 2, G, 32, dk, device=DEV, dtype=BF)
+        vc = torch.zeros(nb + 2, G, 32, dk, device=DEV, dtype=BF)
+        us = timed(lambda: ops.norm_kv_store(conv, pos, kc, vc, slots, Hq, G, dk, dk, 1e-5, True, True,
+                                             (0.5, 1024), BF), reps)
+        emit("norm_kv_store", name, us, gbytes=T * C * 6 / 1e9, like="rope_kv_store")
+        rope = ref.rope_table(64, 1024, 1e4).to(DEV)
+        us = timed(lambda: ops.rope_kv_store(aproj[:, :C], pos, rope, kc, vc, slots, Hq, G, dk, dk), reps)
+        emit("rope_kv_store (same heads)", name, us, gbytes=T * C * 4 / 1e9)
+        # selective scan: 2048 channels of 16 states, 4 taps, gate in the epilogue
+        I, N = W, 16
+        xw, xb = torch.randn(I, K, device=DEV) * 0.3, torch.randn(I, device=DEV) * 0.1
+        xst = torch.zeros(n, K - 1, I, device=DEV)
+        us = timed(lambda: ops.causal_conv(aproj[:, C: C + I], xw, xb, xst, m, True, BF), reps)
+        emit("causal_conv (x, 4 taps, 16-bit out)", name, us, gbytes=T * I * 4 / 1e9, like="causal_conv")
+        x = torch.randn(T, I, device=DEV, dtype=BF)
+        dt = torch.randn(T, I, device=DEV, dtype=BF)
+        dbc = torch.randn(T, 128 + 2 * N, device=DEV, dtype=BF)
+        At = -(1 + 15 * torch.rand(N, I, device=DEV))
+        dtb, D = torch.randn(I, device=DEV) - 3, torch.ones(I, device=DEV)
+        Ss = torch.zeros(n, N, I, device=DEV)
+        feats = torch.empty(T, 2 * W, device=DEV, dtype=BF)
+        us = timed(lambda: ops.selective_scan(x, dt, dbc[:, 128:], At, dtb, D, aproj[:, C + I:], Ss, m,
+                                              1.0, feats[:, W:]), reps)
+        emit("selective_scan (+ gate)", name, us, gbytes=(2 * n * N * I * 4 + T * I * 8) / 1e9,
+             tflop=6 * T * N * I / 1e12, like="ssd_scan")
+        # feed-forwards: PolyNorm on 8256 columns, clamped gated experts of 2752, routing over 9
+        z = torch.randn(T, 8256, device=DEV, dtype=BF)
+        coef = torch.tensor([1.0, 0.3, 0.1, 0.0], device=DEV)
+        us = timed(lambda: ops.polynorm(z, coef, 1e-5), reps)
+        emit("polynorm", f"{T}x8256", us, gbytes=T * 8256 * 4 / 1e9, like="relu_sq")
+        us = timed(lambda: ops.relu_sq(z), reps)
+        emit("relu_sq (same shape)", f"{T}x8256", us, gbytes=T * 8256 * 4 / 1e9)
+        gu = torch.randn(2 * T, 2 * 2752, device=DEV, dtype=BF)
+        us = timed(lambda: ops.swiglu_clamp(gu, 7.0), reps)
+        emit("swiglu_clamp", f"{2 * T}x2752", us, gbytes=2 * T * 2752 * 6 / 1e9, like="silu_mul")
+        us = timed(lambda: ops.silu_mul(gu), reps)
+        emit("silu_mul (same shape)", f"{2 * T}x2752", us, gbytes=2 * T * 2752 * 6 / 1e9)
+        logits = torch.randn(T, 9, device=DEV)
+        corr = torch.randn(9, device=DEV) * 0.01
+        us = timed(lambda: ops.moe_route_softmax_all(logits, corr, 2, 8), reps)
+        emit("moe_route_softmax_all", f"{T}x9", us, like="moe_topk_softmax")
+        us = timed(lambda: ops.moe_topk_softmax(logits[:, :8].contiguous(), 2), reps)
+        emit("moe_topk_softmax (8 experts)", f"{T}x8", us)
+        ids = torch.randint(0, 32000, (T,), device=DEV)
+        tab = torch.randn(32000, W, device=DEV, dtype=BF)
+        ptab = torch.randn(8192, W, device=DEV)
+        xs = torch.empty(T, W, device=DEV)
+        us = timed(lambda: ops.embed_pos(ids, pos, tab, 45.0, ptab, xs), reps)
+        emit("embed_pos", f"{T}x{W}", us, gbytes=T * W * 10 / 1e9)
+
+
 if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--reps", type=int, default=20)
@@ -368,4 +456,4 @@ if __name__ == "__main__":
     ops.load_extension(strict=True)
     for part in a.only.split(","):
         {"attention": attention, "recurrent": recurrent, "rows": rows, "konovik": konovik,
-         "nolesun": nolesun}[part](a.reps)
+         "nolesun": nolesun, "lorenex": lorenex}[part](a.reps)
