@@ -763,7 +763,7 @@ def _lorenex_spec(entry: dict, rank: Optional[int]) -> MixerSpec:
     H = int(l["heads"])
     left = MixerSpec("attention", H, int(l["dim"]), int(l["vdim"]),
                      kv_heads=int(l.get("kv_heads", H)), scale=float(l["scale"]), bias=True,
-                     out_bias=False, conv=int(l.get("conv", 1)), qk_unit=True, v_unit=True,
+                     out_bias=False, conv=int(l.get("conv", 0)), qk_unit=True, v_unit=True,
                      q_temp=(float(qt["coef"]), int(qt["every"])) if qt else None)
     if left.heads % left.kv_heads:
         raise ValueError("heads must be a multiple of the key/value heads")
@@ -800,7 +800,8 @@ def lorenex_config(d: dict, name: str, shapes: Optional[dict] = None) -> ModelCo
     return ModelConfig(
         name, "lorenex", len(specs), int(d["width"]), a.heads, a.kv_heads or a.heads, a.dim,
         max((sp.ff for sp in specs), default=0), int(d["vocab"]),
-        max_position=int(d.get("max_positions", 8192)), rms_eps=float(d["norm"]["eps"]),
+        max_position=int(d.get("max_positions") or (shapes or {}).get("pos", (8192,))[0]),
+        rms_eps=float(d["norm"]["eps"]),
         tie_embeddings=True, learned_pos=True, layer_specs=tuple(specs),
         embed_scale=float(d.get("embedding", {}).get("scale", 1.0)),
         residual_mult=float(d.get("residual_mult", 1.0)), weights_of=share,

@@ -99,7 +99,8 @@ def left_mixer(h, W, p, m, eps):
     H, G, d, dv = m["heads"], m.get("kv_heads", m["heads"]), m["dim"], m["vdim"]
 
     def proj(n):
-        return causal_conv(h @ W[p + n].T + W[p + n + ".b"], W[p + n + ".conv"])
+        u = h @ W[p + n].T + W[p + n + ".b"]
+        return causal_conv(u, W[p + n + ".conv"]) if m.get("conv") else u
     q = rms(proj("q").reshape(T, H, d), eps) * query_temperature(T, m.get("q_temp"))[:, None, None]
     k = rms(proj("k").reshape(T, G, d), eps)
     v = rms(proj("v").reshape(T, G, dv), eps)
@@ -246,7 +247,8 @@ def random_weights(cfg: dict, seed: int = 0, bf16=True) -> dict:
             for n, c in (("q", H * d), ("k", G * d), ("v", G * dv)):
                 put(p + f"mix.left.{n}", c, Wd)
                 put(p + f"mix.left.{n}.b", c, std=0.3)
-                put(p + f"mix.left.{n}.conv", c, l["conv"], std=0.5)
+                if l.get("conv"):
+                    put(p + f"mix.left.{n}.conv", c, l["conv"], std=0.5)
             put(p + "mix.left.o", Wd, H * dv)
             I, N, R = rr["inner"], rr["state"], rr["dt_rank"]
             put(p + "mix.right.in", 2 * I, Wd)

@@ -40,8 +40,11 @@ def gla(heads=2, dim=12, vdim=10, tau=4.0, rank=5):
 
 
 def att(heads=4, kv=2, dim=12, vdim=10, conv=3, scale=0.6, coef=0.5, every=16):
-    return {"heads": heads, "kv_heads": kv, "dim": dim, "vdim": vdim, "conv": conv, "scale": scale,
-            "q_temp": {"coef": coef, "every": every}}
+    m = {"heads": heads, "kv_heads": kv, "dim": dim, "vdim": vdim, "conv": conv, "scale": scale,
+         "q_temp": {"coef": coef, "every": every}}
+    if not conv:
+        del m["conv"]                    # no convolution on q, k and v at all
+    return m
 
 
 def ssm(inner=24, state=6, dt_rank=3, conv=3):
@@ -78,7 +81,8 @@ MIXED = config([glal(gla(), dense()), par(att(), ssm(), moe()),
                     ssm(inner=20, state=9, dt_rank=1, conv=4), dense(40), ls=0.7, rs=1.3),
                 glal(gla(heads=3, dim=8, vdim=16, tau=16.0, rank=2), moe(top=3, identity=2))])
 # values a model may make equal or 1, and parts it may leave out: one head, one state, one
-# expert used of two, no identity expert, no feed-forward, a convolution of one tap and of two,
+# expert used of two, no identity expert, no feed-forward, a convolution of one tap, of two and
+# none,
 # scales and the residual multiplier 1, a query factor that steps at every position, value
 # size = key size, a layer that runs with the weights of one that itself names another, the
 # parallel layer first
@@ -90,7 +94,7 @@ PLAIN = config([par(att(heads=1, kv=1, dim=16, vdim=16, conv=1, scale=1.0, coef=
                 glal(gla(heads=2, dim=8, vdim=8, tau=2.0, rank=3)),
                 par(att(heads=1, kv=1, dim=16, vdim=16, conv=1, scale=1.0, coef=0.25, every=1),
                     ssm(inner=16, state=1, dt_rank=1, conv=1), dense(32), ls=1.0, rs=1.0, weights_of=2),
-                par(att(heads=2, kv=2, dim=8, vdim=8, conv=2, scale=0.7, coef=0.0, every=3),
+                par(att(heads=2, kv=2, dim=8, vdim=8, conv=0, scale=0.7, coef=0.0, every=3),
                     ssm(inner=8, state=4, dt_rank=2, conv=2))],
                width=48, vocab=96, scale=1.0, mult=1.0)
 # sizes the matrix-core prefill kernel, the 16-byte decode paths and the grouped expert GEMM

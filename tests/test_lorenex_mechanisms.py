@@ -295,6 +295,7 @@ def attention_want(q, k, v, H, G, dk, dv, scale, qt, eps=1e-5):
 @pytest.mark.parametrize("dev", DEV)
 @pytest.mark.parametrize("H,G,dk,dv,qt", [(4, 2, 12, 10, (0.5, 16)), (2, 2, 16, 8, (1.5, 1)),
                                           (3, 1, 10, 6, None), (8, 2, 64, 32, (0.3, 7)),
+                                          (4, 2, 48, 40, (0.5, 16)),
                                           (2, 1, 70, 130, (0.5, 1000))])
 def test_unit_norm_attention_and_portions(dev, H, G, dk, dv, qt):
     dev = dev_of(dev)
