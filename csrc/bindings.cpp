@@ -1722,9 +1722,10 @@ void norm_kv_store(Tensor qkv, Tensor positions, Tensor q_out, Tensor k_cache, T
                    Tensor slots, int64_t H, int64_t G, int64_t dk, int64_t dv, double eps,
                    bool qk_unit, bool v_unit, double coef, int64_t every) {
   check_gpu(qkv, "qkv");
-  check_f32(qkv, "qkv");
   c10::hip::HIPGuardMasqueradingAsCUDA g(qkv.device());
-  TORCH_CHECK(qkv.dim() == 2 && qkv.stride(1) == 1 && qkv.size(1) >= (H + G) * dk + G * dv &&
+  // rows may be a column slice of a wider fp32 matrix: the kernel walks them by their stride
+  TORCH_CHECK(qkv.scalar_type() == at::kFloat && qkv.dim() == 2 && qkv.stride(1) == 1 &&
+              qkv.size(1) >= (H + G) * dk + G * dv &&
               H >= 1 && G >= 1 && dk >= 1 && dv >= 1 && every >= 1,
               "kgc.norm_kv_store: qkv fp32 [T, H dk + G dk + G dv]");
   const int64_t T = qkv.size(0);
