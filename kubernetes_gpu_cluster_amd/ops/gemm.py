@@ -705,7 +705,7 @@ _DG_REFINE_ROUNDS = int(os.environ.get("KGC_DGEMM_REFINE_ROUNDS", "5"))
 
 def _dg_candidates(M: int, N: int, K: int, kind: str, packed: bool):
     # (K9v / K9r, measured slower than K9m on every M = 256 shape, are not in the engine's
-    # library: tools/research/; profiles/README.md "Round 3: K9r" / "Round 3: K9v")
+    # library: their sources are under tools/research/)
     from . import _k
     # 11-14: packed 64 / 80 / 112-wide column tiles (gemm_decode.hip kCfg) for the narrow
     # shards of a TP = 8 rank

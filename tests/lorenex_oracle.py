@@ -10,8 +10,6 @@ with rms(v) = v / sqrt(mean(v^2) + eps).  The sublayers read x itself.
 """
 from __future__ import annotations
 
-import math
-
 import numpy as np
 
 
@@ -29,10 +27,6 @@ def silu(z):
 
 def softplus(z):
     return np.logaddexp(0.0, z)
-
-
-def gelu_tanh(z):
-    return 0.5 * z * (1.0 + np.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z ** 3)))
 
 
 def causal_conv(u, w, bias=None):
