@@ -191,6 +191,36 @@ def test_selective_scan_over_steps(dev, I, N):
 
 
 @pytest.mark.parametrize("dev", DEV)
+def test_selective_scan_keeps_and_forgets_per_channel(dev):
+    """Channel 0 has A ~ 0 (its state never decays) and channel 1 a large |A| (it forgets at
+    once): 300 tokens after the only input, channel 0 still returns it, channel 1 returns only
+    the current token's -- in one prompt, in decode rows and in two-token portions."""
+    dev = dev_of(dev)
+    n, I, N = 300, 2, 1
+    x = np.zeros((n, I))
+    x[0] = [1.0, 1.0]
+    x[-1] = [0.0, 2.0]
+    dt = np.ones((n, I))
+    step = oracle.softplus(1.0)
+    bc = np.ones((n, 2 * N))
+    z = np.full((n, I), 30.0)                     # silu(30) = 30
+    At = f32(np.array([[-1e-9, -50.0]]), dev)
+    zero = torch.zeros(I, device=dev)
+    t = {k: f32(a, dev) for k, a in dict(x=x, dt=dt, bc=bc, z=z).items()}
+    for cuts in ([n], [n - 40, 1], [7, 2]):
+        state = torch.full((3, N, I), 5.0, device=dev)
+        out = torch.zeros(n, I, device=dev)
+
+        def fn(lo, hi, m):
+            ops.selective_scan(t["x"][lo:hi], t["dt"][lo:hi], t["bc"][lo:hi], At, zero, zero,
+                               t["z"][lo:hi], state, m, 1.0, out[lo:hi])
+            return out[lo:hi]
+        got = over_steps(n, cuts, dev, fn)
+        np.testing.assert_allclose(got[n - 2], [30.0 * step, 0.0], rtol=1e-5, atol=1e-5)
+        np.testing.assert_allclose(got[n - 1], [30.0 * step, 60.0 * step], rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("dev", DEV)
 def test_scans_in_a_batch_with_padding_rows(dev):
     """Two prompts' portions and three decode rows (one a padding row of slot -1) in one
     step, against each sequence alone; slots handed out in no particular order."""
